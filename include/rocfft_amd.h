@@ -1,0 +1,37 @@
+/*
+ * rocfft_amd.h -- entry points this library adds to the rocfft.h interface.
+ * They have no counterpart in the reference.
+ */
+#ifndef ROCFFT_AMD_H
+#define ROCFFT_AMD_H
+
+#include "rocfft/rocfft.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Plans a transform exactly as rocfft_plan_create would, without touching a
+ * device, and writes the pass list as text (the same text rocfft_plan_get_print
+ * prints; reference rocfft.h:443 / library/src/plan.cpp:4476-4514 is the
+ * nearest counterpart).  text may be NULL.  work_buffer_bytes, when not NULL,
+ * receives what rocfft_plan_get_work_buffer_size would report.  Returns the
+ * status rocfft_plan_create would return for the same arguments, apart from
+ * device errors.
+ */
+ROCFFT_EXPORT rocfft_status rocfft_amd_plan_describe(rocfft_result_placement       placement,
+                                                     rocfft_transform_type         transform_type,
+                                                     rocfft_precision              precision,
+                                                     size_t                        dimensions,
+                                                     const size_t*                 lengths,
+                                                     size_t                        number_of_transforms,
+                                                     const rocfft_plan_description description,
+                                                     char*                         text,
+                                                     size_t                        text_len,
+                                                     size_t*                       work_buffer_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

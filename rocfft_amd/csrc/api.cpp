@@ -1,0 +1,659 @@
+// api.cpp -- the rocfft.h entry points: handles, defaults, validation, plan
+// creation and execution.  Behaviour follows the reference API glue
+// (library/src/plan.cpp:69-77, :87-197, :224-285, :397-488, :729-779, :2959-3145,
+// :3279-3289; library/src/transform.cpp:35-103, :331-474); the planner behind it
+// is this library's own (plan.cpp).
+#include "gpu_rt.h"
+#include "plan.h"
+#include "rocfft/rocfft.h"
+#include "rocfft_amd.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+using namespace fftamd;
+
+#define ROCFFT_AMD_VERSION "1.0.32.amd-gfx950-0.1"
+
+struct rocfft_plan_description_t
+{
+    rocfft_array_type   inArrayType  = rocfft_array_type_unset;
+    rocfft_array_type   outArrayType = rocfft_array_type_unset;
+    std::vector<size_t> inStrides, outStrides;
+    size_t              inDist = 0, outDist = 0;
+    size_t              inOffset[2]  = {0, 0};
+    size_t              outOffset[2] = {0, 0};
+    double              scale        = 1.0;
+    bool                has_scale    = false;
+    bool                distributed  = false; // a field or communicator was attached
+};
+
+struct rocfft_plan_t
+{
+    Problem     prob;
+    ExecPlan    exec;
+    int         device = 0;
+    std::string error;
+};
+
+struct rocfft_execution_info_t
+{
+    void*  workBuffer     = nullptr;
+    size_t workBufferSize = 0;
+    void*  stream         = nullptr;
+};
+
+struct rocfft_field_t
+{
+    int bricks = 0;
+};
+struct rocfft_brick_t
+{
+    int device = 0;
+};
+
+// ---------------------------------------------------------------------------
+// defaults and validation
+
+// fills unset array types, strides and distances (reference plan.cpp:87-197)
+static void init_defaults(rocfft_plan_description_t& d, rocfft_transform_type type,
+                          rocfft_result_placement placement, const std::vector<size_t>& lengths,
+                          const std::vector<size_t>& outputLengths)
+{
+    const size_t rank = lengths.size();
+    if(d.inArrayType == rocfft_array_type_unset)
+    {
+        if(type == rocfft_transform_type_real_forward)
+            d.inArrayType = rocfft_array_type_real;
+        else if(type == rocfft_transform_type_real_inverse)
+            d.inArrayType = rocfft_array_type_hermitian_interleaved;
+        else
+            d.inArrayType = rocfft_array_type_complex_interleaved;
+    }
+    if(d.outArrayType == rocfft_array_type_unset)
+    {
+        if(type == rocfft_transform_type_real_forward)
+            d.outArrayType = rocfft_array_type_hermitian_interleaved;
+        else if(type == rocfft_transform_type_real_inverse)
+            d.outArrayType = rocfft_array_type_real;
+        else
+            d.outArrayType = rocfft_array_type_complex_interleaved;
+    }
+    const bool inplace = placement == rocfft_placement_inplace;
+    if(d.inStrides.empty())
+    {
+        d.inStrides.push_back(1);
+        if(type == rocfft_transform_type_real_forward && inplace)
+        {
+            // rows padded so that the Hermitian output fits over the real input
+            size_t dist = 2 * outputLengths[0];
+            for(size_t i = 1; i < rank; ++i)
+            {
+                d.inStrides.push_back(dist);
+                dist *= lengths[i];
+            }
+        }
+        else
+            for(size_t i = 1; i < rank; ++i)
+                d.inStrides.push_back(lengths[i - 1] * d.inStrides[i - 1]);
+    }
+    if(d.outStrides.empty())
+    {
+        d.outStrides.push_back(1);
+        if(type == rocfft_transform_type_real_inverse && inplace)
+        {
+            size_t dist = 2 * lengths[0];
+            for(size_t i = 1; i < rank; ++i)
+            {
+                d.outStrides.push_back(dist);
+                dist *= lengths[i];
+            }
+        }
+        else
+            for(size_t i = 1; i < rank; ++i)
+                d.outStrides.push_back(outputLengths[i - 1] * d.outStrides[i - 1]);
+    }
+    if(d.inDist == 0)
+    {
+        if(type == rocfft_transform_type_real_forward && rank == 1 && inplace)
+            d.inDist = 2 * (lengths[0] / 2 + 1) * d.inStrides[0];
+        else
+            d.inDist = lengths[rank - 1] * d.inStrides[rank - 1];
+    }
+    if(d.outDist == 0)
+    {
+        if(type == rocfft_transform_type_real_inverse && rank == 1 && inplace)
+            d.outDist = 2 * lengths[0] * d.outStrides[0];
+        else
+            d.outDist = outputLengths[rank - 1] * d.outStrides[rank - 1];
+    }
+}
+
+// transform type, array types and placement must agree (reference plan.cpp:729-779)
+static rocfft_status check_array_types(rocfft_transform_type type, rocfft_result_placement placement,
+                                       const rocfft_plan_description_t& d)
+{
+    auto is_complex = [](rocfft_array_type t) {
+        return t == rocfft_array_type_complex_interleaved || t == rocfft_array_type_complex_planar;
+    };
+    auto is_herm = [](rocfft_array_type t) {
+        return t == rocfft_array_type_hermitian_interleaved || t == rocfft_array_type_hermitian_planar;
+    };
+    const bool inplace = placement == rocfft_placement_inplace;
+    switch(type)
+    {
+    case rocfft_transform_type_complex_forward:
+    case rocfft_transform_type_complex_inverse:
+        if(!is_complex(d.inArrayType) || !is_complex(d.outArrayType))
+            return rocfft_status_invalid_array_type;
+        if(inplace && d.inArrayType != d.outArrayType)
+            return rocfft_status_invalid_array_type;
+        break;
+    case rocfft_transform_type_real_forward:
+        if(d.inArrayType != rocfft_array_type_real || !is_herm(d.outArrayType))
+            return rocfft_status_invalid_array_type;
+        if(inplace && d.outArrayType != rocfft_array_type_hermitian_interleaved)
+            return rocfft_status_invalid_array_type;
+        break;
+    case rocfft_transform_type_real_inverse:
+        if(d.outArrayType != rocfft_array_type_real || !is_herm(d.inArrayType))
+            return rocfft_status_invalid_array_type;
+        if(inplace && d.inArrayType != rocfft_array_type_hermitian_interleaved)
+            return rocfft_status_invalid_array_type;
+        break;
+    default:
+        return rocfft_status_invalid_arg_value;
+    }
+    return rocfft_status_success;
+}
+
+// Turns the API arguments into a Problem (dimension order as given; the planner
+// picks its own pass order, so the reference's stride sort, plan.cpp:224-285, is
+// only applied to drop unit-length trailing dimensions).
+static rocfft_status make_problem(Problem& p, rocfft_result_placement placement,
+                                  rocfft_transform_type type, rocfft_precision precision,
+                                  size_t dimensions, const size_t* lengths, size_t batch,
+                                  const rocfft_plan_description description)
+{
+    if(dimensions < 1 || dimensions > 3)
+        return rocfft_status_invalid_dimensions;
+    if(!lengths)
+        return rocfft_status_failure;
+    if((int)type < 0 || (int)type > 3)
+        return rocfft_status_invalid_arg_value;
+    std::vector<size_t> len(lengths, lengths + dimensions);
+    for(size_t v : len)
+        if(v == 0)
+            return rocfft_status_invalid_dimensions;
+    const bool is_real
+        = type == rocfft_transform_type_real_forward || type == rocfft_transform_type_real_inverse;
+    // array lengths on each side (reference plan.cpp:2980-2987)
+    std::vector<size_t> ilen = len, olen = len;
+    if(type == rocfft_transform_type_real_forward)
+        olen[0] = len[0] / 2 + 1;
+    if(type == rocfft_transform_type_real_inverse)
+        ilen[0] = len[0] / 2 + 1;
+    rocfft_plan_description_t d;
+    if(description)
+        d = *description;
+    if(d.distributed)
+        return rocfft_status_failure;
+    if(!d.inStrides.empty() && d.inStrides.size() != dimensions)
+        return rocfft_status_invalid_strides;
+    if(!d.outStrides.empty() && d.outStrides.size() != dimensions)
+        return rocfft_status_invalid_strides;
+    init_defaults(d, type, placement, ilen, olen);
+    rocfft_status st = check_array_types(type, placement, d);
+    if(st != rocfft_status_success)
+        return st;
+    (void)is_real;
+    memset(&p, 0, sizeof(p));
+    p.type      = type;
+    p.precision = precision;
+    p.placement = placement;
+    p.rank      = dimensions;
+    p.batch     = batch;
+    p.in_type   = d.inArrayType;
+    p.out_type  = d.outArrayType;
+    for(size_t i = 0; i < dimensions; ++i)
+    {
+        p.len[i]     = len[i];
+        p.istride[i] = d.inStrides[i];
+        p.ostride[i] = d.outStrides[i];
+    }
+    p.idist = d.inDist;
+    p.odist = d.outDist;
+    for(int i = 0; i < 2; ++i)
+    {
+        p.ioffset[i] = d.inOffset[i];
+        p.ooffset[i] = d.outOffset[i];
+    }
+    p.scale     = d.scale;
+    p.has_scale = d.has_scale && d.scale != 1.0;
+    // trailing unit dimensions carry no work (reference plan.cpp:271-276)
+    while(p.rank > 1 && p.len[p.rank - 1] == 1)
+        --p.rank;
+    return rocfft_status_success;
+}
+
+// ---------------------------------------------------------------------------
+// entry points
+
+static int  g_setup_count = 0;
+static bool g_log_plan    = false;
+
+extern "C" {
+
+rocfft_status rocfft_setup(void)
+{
+    ++g_setup_count;
+    const char* layer = getenv("ROCFFT_LAYER");
+    // bit 3 of ROCFFT_LAYER asks for the plan log (reference logging.h:139-150)
+    g_log_plan = layer && (atoi(layer) & 8);
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_cleanup(void)
+{
+    if(g_setup_count > 0)
+        --g_setup_count;
+    table_cache_clear();
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement placement,
+                                 rocfft_transform_type transform_type, rocfft_precision precision,
+                                 size_t dimensions, const size_t* lengths, size_t number_of_transforms,
+                                 const rocfft_plan_description description)
+{
+    if(!plan)
+        return rocfft_status_failure;
+    *plan = nullptr;
+    try
+    {
+        rocfft_plan_t* p  = new rocfft_plan_t;
+        rocfft_status  st = make_problem(p->prob, placement, transform_type, precision, dimensions,
+                                        lengths, number_of_transforms, description);
+        if(st == rocfft_status_success)
+        {
+            int ndev = 0;
+            if(fftrt_device_count(&ndev) != 0 || ndev < 1)
+            {
+                p->error = "no GPU available";
+                st       = rocfft_status_failure;
+            }
+        }
+        if(st == rocfft_status_success)
+        {
+            fftrt_device_info(&p->device, nullptr, nullptr, nullptr, 0);
+            st = build_exec_plan(p->prob, p->exec, false, p->error);
+        }
+        if(st != rocfft_status_success)
+        {
+            if(getenv("ROCFFT_AMD_VERBOSE") && !p->error.empty())
+                fprintf(stderr, "rocfft_plan_create: %s\n", p->error.c_str());
+            delete p;
+            return st;
+        }
+        if(g_log_plan)
+            fputs(p->exec.describe().c_str(), stderr);
+        *plan = p;
+        return rocfft_status_success;
+    }
+    catch(...)
+    {
+        return rocfft_status_failure;
+    }
+}
+
+rocfft_status rocfft_execute(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
+                             rocfft_execution_info info)
+{
+    if(!plan || !in_buffer || !in_buffer[0])
+        return rocfft_status_failure;
+    try
+    {
+        const ExecPlan& ep     = plan->exec;
+        const Problem&  pr     = plan->prob;
+        auto            planar = [](rocfft_array_type t) {
+            return t == rocfft_array_type_complex_planar || t == rocfft_array_type_hermitian_planar;
+        };
+        void* in[2]  = {in_buffer[0], planar(pr.in_type) ? in_buffer[1] : nullptr};
+        void* out[2] = {nullptr, nullptr};
+        if(ep.inplace)
+        {
+            out[0] = in[0];
+            out[1] = in[1];
+        }
+        else
+        {
+            if(!out_buffer || !out_buffer[0])
+                return rocfft_status_failure;
+            out[0] = out_buffer[0];
+            out[1] = planar(pr.out_type) ? out_buffer[1] : nullptr;
+        }
+        if((planar(pr.in_type) && !in[1]) || (planar(pr.out_type) && !out[1]))
+            return rocfft_status_failure;
+        void*  stream = info ? info->stream : nullptr;
+        size_t need   = ep.work_bytes();
+        void*  work   = nullptr;
+        bool   own    = false;
+        if(need)
+        {
+            if(info && info->workBuffer)
+            {
+                if(info->workBufferSize < need)
+                    return rocfft_status_invalid_work_buffer;
+                work = info->workBuffer;
+            }
+            else
+            {
+                // no caller-owned scratch: allocate for this call (reference
+                // transform.cpp:424-434); impossible while the stream is being captured
+                if(fftrt_stream_capturing(stream))
+                    return rocfft_status_invalid_work_buffer;
+                if(fftrt_malloc(&work, need) != 0)
+                    return rocfft_status_failure;
+                own = true;
+            }
+        }
+        rocfft_status st = run_exec_plan(ep, in, out, work, stream);
+        if(own)
+        {
+            fftrt_stream_sync(stream);
+            fftrt_free(work);
+        }
+        return st;
+    }
+    catch(...)
+    {
+        return rocfft_status_failure;
+    }
+}
+
+rocfft_status rocfft_plan_destroy(rocfft_plan plan)
+{
+    delete plan;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_description_set_scale_factor(rocfft_plan_description description,
+                                                       const double            scale_factor)
+{
+    if(!description)
+        return rocfft_status_failure;
+    if(!std::isfinite(scale_factor))
+        return rocfft_status_invalid_arg_value;
+    description->scale     = scale_factor;
+    description->has_scale = true;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_description_set_data_layout(rocfft_plan_description description,
+                                                      const rocfft_array_type in_array_type,
+                                                      const rocfft_array_type out_array_type,
+                                                      const size_t*           in_offsets,
+                                                      const size_t*           out_offsets,
+                                                      const size_t            in_strides_size,
+                                                      const size_t*           in_strides,
+                                                      const size_t            in_distance,
+                                                      const size_t            out_strides_size,
+                                                      const size_t*           out_strides,
+                                                      const size_t            out_distance)
+{
+    if(!description)
+        return rocfft_status_failure;
+    auto planar = [](rocfft_array_type t) {
+        return t == rocfft_array_type_complex_planar || t == rocfft_array_type_hermitian_planar;
+    };
+    description->inArrayType  = in_array_type;
+    description->outArrayType = out_array_type;
+    if(in_offsets)
+    {
+        description->inOffset[0] = in_offsets[0];
+        if(planar(in_array_type))
+            description->inOffset[1] = in_offsets[1];
+    }
+    if(out_offsets)
+    {
+        description->outOffset[0] = out_offsets[0];
+        if(planar(out_array_type))
+            description->outOffset[1] = out_offsets[1];
+    }
+    if(in_strides)
+        description->inStrides.assign(in_strides, in_strides + in_strides_size);
+    if(in_distance)
+        description->inDist = in_distance;
+    if(out_strides)
+        description->outStrides.assign(out_strides, out_strides + out_strides_size);
+    if(out_distance)
+        description->outDist = out_distance;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_field_create(rocfft_field* field)
+{
+    if(!field)
+        return rocfft_status_failure;
+    *field = new rocfft_field_t;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_field_destroy(rocfft_field field)
+{
+    delete field;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_get_version_string(char* buf, size_t len)
+{
+    static const char v[] = ROCFFT_AMD_VERSION;
+    if(!buf)
+        return rocfft_status_failure;
+    if(len < sizeof(v))
+        return rocfft_status_invalid_arg_value;
+    memcpy(buf, v, sizeof(v));
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_description_set_comm(rocfft_plan_description description,
+                                               rocfft_comm_type comm_type, void* comm_handle)
+{
+    (void)comm_handle;
+    if(!description)
+        return rocfft_status_failure;
+    if(comm_type != rocfft_comm_none)
+        description->distributed = true;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_brick_create(rocfft_brick* brick, const size_t* field_lower,
+                                  const size_t* field_upper, const size_t* brick_stride, size_t dim,
+                                  int deviceID)
+{
+    if(!brick || !field_lower || !field_upper || !brick_stride || dim == 0)
+        return rocfft_status_failure;
+    *brick           = new rocfft_brick_t;
+    (*brick)->device = deviceID;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_brick_destroy(rocfft_brick brick)
+{
+    delete brick;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_field_add_brick(rocfft_field field, rocfft_brick brick)
+{
+    if(!field || !brick)
+        return rocfft_status_failure;
+    ++field->bricks;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_plan_description_add_infield(rocfft_plan_description description,
+                                                  rocfft_field            field)
+{
+    if(!description || !field)
+        return rocfft_status_failure;
+    description->distributed = true;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_plan_description_add_outfield(rocfft_plan_description description,
+                                                   rocfft_field            field)
+{
+    if(!description || !field)
+        return rocfft_status_failure;
+    description->distributed = true;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_get_work_buffer_size(const rocfft_plan plan, size_t* size_in_bytes)
+{
+    if(!plan || !size_in_bytes)
+        return rocfft_status_failure;
+    *size_in_bytes = plan->exec.work_bytes();
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_get_print(const rocfft_plan plan)
+{
+    if(!plan)
+        return rocfft_status_failure;
+    fputs(plan->exec.describe().c_str(), stdout);
+    fflush(stdout);
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_plan_description_create(rocfft_plan_description* description)
+{
+    if(!description)
+        return rocfft_status_failure;
+    *description = new rocfft_plan_description_t;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_plan_description_destroy(rocfft_plan_description description)
+{
+    delete description;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_execution_info_create(rocfft_execution_info* info)
+{
+    if(!info)
+        return rocfft_status_failure;
+    *info = new rocfft_execution_info_t;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_execution_info_destroy(rocfft_execution_info info)
+{
+    delete info;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_execution_info_set_work_buffer(rocfft_execution_info info, void* work_buffer,
+                                                    const size_t size_in_bytes)
+{
+    if(!info)
+        return rocfft_status_failure;
+    if(!work_buffer)
+        return rocfft_status_invalid_work_buffer;
+    info->workBuffer     = work_buffer;
+    info->workBufferSize = size_in_bytes;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_execution_info_set_stream(rocfft_execution_info info, void* stream)
+{
+    if(!info)
+        return rocfft_status_failure;
+    info->stream = stream;
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_execution_info_set_load_callback(rocfft_execution_info info, void** cb_functions,
+                                                      void** cb_data, size_t shared_mem_bytes)
+{
+    (void)cb_data;
+    if(!info)
+        return rocfft_status_failure;
+    if(shared_mem_bytes)
+        return rocfft_status_invalid_arg_value;
+    // clearing a callback is a no-op; installing one needs run-time compiled kernels
+    if(!cb_functions || !cb_functions[0])
+        return rocfft_status_success;
+    return rocfft_status_failure;
+}
+rocfft_status rocfft_execution_info_set_store_callback(rocfft_execution_info info, void** cb_functions,
+                                                       void** cb_data, size_t shared_mem_bytes)
+{
+    (void)cb_data;
+    if(!info)
+        return rocfft_status_failure;
+    if(shared_mem_bytes)
+        return rocfft_status_invalid_arg_value;
+    if(!cb_functions || !cb_functions[0])
+        return rocfft_status_success;
+    return rocfft_status_failure;
+}
+
+rocfft_status rocfft_cache_serialize(void** buffer, size_t* buffer_len_bytes)
+{
+    if(!buffer || !buffer_len_bytes)
+        return rocfft_status_failure;
+    *buffer           = malloc(1);
+    *buffer_len_bytes = 0;
+    return rocfft_status_success;
+}
+rocfft_status rocfft_cache_buffer_free(void* buffer)
+{
+    free(buffer);
+    return rocfft_status_success;
+}
+rocfft_status rocfft_cache_deserialize(const void* buffer, size_t buffer_len_bytes)
+{
+    (void)buffer_len_bytes;
+    if(!buffer)
+        return rocfft_status_failure;
+    return rocfft_status_success;
+}
+
+// ---------------------------------------------------------------------------
+// extension: plan description without touching a device
+
+rocfft_status rocfft_amd_plan_describe(rocfft_result_placement placement,
+                                       rocfft_transform_type transform_type, rocfft_precision precision,
+                                       size_t dimensions, const size_t* lengths,
+                                       size_t number_of_transforms,
+                                       const rocfft_plan_description description, char* text,
+                                       size_t text_len, size_t* work_buffer_bytes)
+{
+    try
+    {
+        Problem       prob;
+        rocfft_status st = make_problem(prob, placement, transform_type, precision, dimensions, lengths,
+                                        number_of_transforms, description);
+        if(st != rocfft_status_success)
+            return st;
+        ExecPlan    ep;
+        std::string err;
+        st = build_exec_plan(prob, ep, true, err);
+        std::string out = st == rocfft_status_success ? ep.describe() : ("error: " + err + "\n");
+        if(text && text_len)
+        {
+            size_t ncopy = std::min(text_len - 1, out.size());
+            memcpy(text, out.data(), ncopy);
+            text[ncopy] = 0;
+        }
+        if(work_buffer_bytes)
+            *work_buffer_bytes = st == rocfft_status_success ? ep.work_bytes() : 0;
+        return st;
+    }
+    catch(...)
+    {
+        return rocfft_status_failure;
+    }
+}
+}

@@ -1,0 +1,46 @@
+// gpu_rt.h -- the thin C-ABI layer between the host library (planner, API,
+// table builders: plain C++) and the GPU (HIP runtime calls and kernel
+// launches).  Nothing above this layer includes a HIP header.
+//
+// Two implementations exist: kernels.hip (the product, HIP on gfx950) and
+// tests/emu/gpu_rt_emu.cpp (host loops over the same kernel bodies, used only
+// by the CPU test-suite to exercise the planner without a GPU).
+#ifndef ROCFFT_AMD_GPU_RT_H
+#define ROCFFT_AMD_GPU_RT_H
+
+#include "kparams.h"
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// 0 on success, non-zero (the HIP error code) otherwise
+int fftrt_device_count(int* count);
+int fftrt_device_info(int* device, int* compute_units, int* lds_bytes, char* arch, size_t arch_len);
+int fftrt_malloc(void** ptr, size_t bytes);
+int fftrt_free(void* ptr);
+int fftrt_upload(void* dst, const void* src, size_t bytes);
+int fftrt_download(void* dst, const void* src, size_t bytes);
+int fftrt_stream_sync(void* stream);
+int fftrt_device_sync(void);
+// 1 when `stream` is being captured into a graph
+int fftrt_stream_capturing(void* stream);
+
+// precision: 0 = float, 1 = double.  vec: 1 when both sides are interleaved
+// complex and can move (re, im) pairs with one access.
+int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
+                      size_t lds_bytes, void* stream);
+int fftrt_launch_real_post(const struct fftk_real_params* p, int precision, void* stream);
+int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void* stream);
+
+// event timing, used by the optional per-pass profile log
+int fftrt_event_create(void** ev);
+int fftrt_event_destroy(void* ev);
+int fftrt_event_record(void* ev, void* stream);
+int fftrt_event_elapsed_ms(void* start, void* stop, float* ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,246 @@
+// kernels.hip -- gfx950 kernels and the HIP side of the C-ABI runtime layer.
+#include "gpu_rt.h"
+#include "tile_core.h"
+#include <hip/hip_runtime.h>
+#include <mutex>
+#include <string.h>
+
+namespace
+{
+
+template <typename T>
+__device__ __forceinline__ void run_passes(const fftk_params&         p,
+                                           typename cplx_of<T>::type* lds,
+                                           uint32_t                   w,
+                                           uint32_t                   tt,
+                                           bool                       active)
+{
+    typedef typename cplx_of<T>::type C;
+    for(uint32_t pass = 0; pass < p.nf; ++pass)
+    {
+        C r[FFTK_REG_ELEMS];
+        switch(p.radix[pass])
+        {
+#define FFTK_CASE(R)                                         \
+    case R:                                                  \
+        pass_read<T, R>(p, lds, w, tt, active, r);           \
+        __syncthreads();                                     \
+        pass_write<T, R>(p, (int)pass, lds, w, tt, active, r); \
+        break;
+            FFTK_CASE(2)
+            FFTK_CASE(3)
+            FFTK_CASE(4)
+            FFTK_CASE(5)
+            FFTK_CASE(7)
+            FFTK_CASE(8)
+            FFTK_CASE(11)
+            FFTK_CASE(13)
+            FFTK_CASE(16)
+#undef FFTK_CASE
+        default:
+            __syncthreads();
+            break;
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T, bool VEC, int BLK>
+__global__ __launch_bounds__(BLK) void tile_fft_kernel(const fftk_params p)
+{
+    typedef typename cplx_of<T>::type C;
+    extern __shared__ double2         smem_raw[];
+    C*                                lds = reinterpret_cast<C*>(smem_raw);
+    const uint32_t                    tid = threadIdx.x;
+    TileCtx<T>                        c;
+    tile_decode<T>(p, blockIdx.x, c);
+    tile_load<T, VEC>(p, c, lds, tid);
+    __syncthreads();
+    uint32_t w, tt;
+    bool     active;
+    thread_role(p, tid, w, tt, active);
+    run_passes<T>(p, lds, w, tt, active);
+    if(p.flags & FFTK_F_CONV)
+    {
+        tile_conv<T>(p, c, lds, tid);
+        __syncthreads();
+        run_passes<T>(p, lds, w, tt, active);
+    }
+    tile_store<T, VEC>(p, c, lds, tid);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void real_post_kernel(const fftk_real_params p)
+{
+    real_post_elem<T>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void real_pre_kernel(const fftk_real_params p)
+{
+    real_pre_elem<T>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+constexpr size_t MAX_LDS_BYTES = 160 * 1024;
+
+template <typename K>
+int raise_lds_limit(K kernel)
+{
+    return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)MAX_LDS_BYTES);
+}
+
+template <typename T, bool VEC, int BLK>
+int launch_tile_t(const fftk_params* p, uint32_t grid, size_t lds_bytes, hipStream_t stream)
+{
+    auto kernel = tile_fft_kernel<T, VEC, BLK>;
+    if(lds_bytes > 64 * 1024)
+    {
+        // raised once per kernel and device; hipFuncSetAttribute is not a
+        // stream operation, so it is legal during graph capture
+        static std::once_flag once[16];
+        int                   dev = 0;
+        (void)hipGetDevice(&dev);
+        int rc = 0;
+        std::call_once(once[dev & 15], [&]() { rc = raise_lds_limit(kernel); });
+        if(rc)
+            return rc;
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p->nthreads), lds_bytes, stream, *p);
+    return (int)hipGetLastError();
+}
+
+template <typename T, bool VEC>
+int launch_tile_b(const fftk_params* p, uint32_t grid, size_t lds_bytes, hipStream_t stream)
+{
+    if(p->nthreads <= 256)
+        return launch_tile_t<T, VEC, 256>(p, grid, lds_bytes, stream);
+    return launch_tile_t<T, VEC, 512>(p, grid, lds_bytes, stream);
+}
+
+} // namespace
+
+extern "C" {
+
+int fftrt_device_count(int* count)
+{
+    return (int)hipGetDeviceCount(count);
+}
+
+int fftrt_device_info(int* device, int* compute_units, int* lds_bytes, char* arch, size_t arch_len)
+{
+    int dev = 0;
+    int rc  = (int)hipGetDevice(&dev);
+    if(rc)
+        return rc;
+    hipDeviceProp_t prop;
+    rc = (int)hipGetDeviceProperties(&prop, dev);
+    if(rc)
+        return rc;
+    if(device)
+        *device = dev;
+    if(compute_units)
+        *compute_units = prop.multiProcessorCount;
+    if(lds_bytes)
+        *lds_bytes = (int)prop.maxSharedMemoryPerMultiProcessor;
+    if(arch && arch_len)
+    {
+        strncpy(arch, prop.gcnArchName, arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    return 0;
+}
+
+int fftrt_malloc(void** ptr, size_t bytes)
+{
+    return (int)hipMalloc(ptr, bytes);
+}
+int fftrt_free(void* ptr)
+{
+    return (int)hipFree(ptr);
+}
+int fftrt_upload(void* dst, const void* src, size_t bytes)
+{
+    return (int)hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice);
+}
+int fftrt_download(void* dst, const void* src, size_t bytes)
+{
+    return (int)hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost);
+}
+int fftrt_stream_sync(void* stream)
+{
+    return (int)hipStreamSynchronize((hipStream_t)stream);
+}
+int fftrt_device_sync(void)
+{
+    return (int)hipDeviceSynchronize();
+}
+int fftrt_stream_capturing(void* stream)
+{
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if(hipStreamIsCapturing((hipStream_t)stream, &st) != hipSuccess)
+        return 0;
+    return st == hipStreamCaptureStatusActive ? 1 : 0;
+}
+
+int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
+                      size_t lds_bytes, void* stream)
+{
+    hipStream_t s = (hipStream_t)stream;
+    if(p->nthreads == 0 || p->nthreads > 512 || (p->nthreads & 63) || lds_bytes > MAX_LDS_BYTES
+       || grid == 0)
+        return (int)hipErrorInvalidValue;
+    if(precision == 0)
+        return vec ? launch_tile_b<float, true>(p, grid, lds_bytes, s)
+                   : launch_tile_b<float, false>(p, grid, lds_bytes, s);
+    return vec ? launch_tile_b<double, true>(p, grid, lds_bytes, s)
+               : launch_tile_b<double, false>(p, grid, lds_bytes, s);
+}
+
+static uint32_t real_grid(const struct fftk_real_params* p)
+{
+    uint64_t total = (uint64_t)(p->half / 2 + 1) * p->rows0 * p->rows1 * p->rows2;
+    return (uint32_t)((total + 255) / 256);
+}
+
+int fftrt_launch_real_post(const struct fftk_real_params* p, int precision, void* stream)
+{
+    uint32_t grid = real_grid(p);
+    if(precision == 0)
+        hipLaunchKernelGGL(real_post_kernel<float>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
+    else
+        hipLaunchKernelGGL(real_post_kernel<double>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
+    return (int)hipGetLastError();
+}
+
+int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void* stream)
+{
+    uint32_t grid = real_grid(p);
+    if(precision == 0)
+        hipLaunchKernelGGL(real_pre_kernel<float>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
+    else
+        hipLaunchKernelGGL(real_pre_kernel<double>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
+    return (int)hipGetLastError();
+}
+
+int fftrt_event_create(void** ev)
+{
+    return (int)hipEventCreate((hipEvent_t*)ev);
+}
+int fftrt_event_destroy(void* ev)
+{
+    return (int)hipEventDestroy((hipEvent_t)ev);
+}
+int fftrt_event_record(void* ev, void* stream)
+{
+    return (int)hipEventRecord((hipEvent_t)ev, (hipStream_t)stream);
+}
+int fftrt_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+    int rc = (int)hipEventSynchronize((hipEvent_t)stop);
+    if(rc)
+        return rc;
+    return (int)hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop);
+}
+}

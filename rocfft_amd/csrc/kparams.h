@@ -1,0 +1,110 @@
+// kparams.h -- launch descriptors shared by the host planner and the device kernels.
+//
+// One "tile pass" is a batch of 1D FFTs of length n.  A workgroup owns a tile of
+// W transforms that are neighbours along the "tile" dimension, stages the tile in
+// LDS, runs every Stockham pass there and writes the tile back.  Whether global
+// accesses run fastest along the transform or along the tile dimension is chosen
+// per side, so the same kernel serves unit-stride rows, strided columns and
+// row-in/column-out (transposing) passes.
+#ifndef ROCFFT_AMD_KPARAMS_H
+#define ROCFFT_AMD_KPARAMS_H
+
+#include <stdint.h>
+
+#define FFTK_MAX_PASSES 12
+#define FFTK_REG_ELEMS 16 // complex values a thread keeps in registers per pass
+
+// how a tile element is fetched
+enum fftk_load_op
+{
+    FFTK_LOAD_COMPLEX     = 0, // (re, im) from in0/in1
+    FFTK_LOAD_REAL        = 1, // re from in0, im = 0
+    FFTK_LOAD_C2R_PRE     = 2, // Hermitian bins -> half-length complex input of the inverse FFT
+    FFTK_LOAD_HERM_EXPAND = 3  // bins 0..n_in/2 plus their conjugate mirror (odd-length real inverse)
+};
+
+// how a tile element is written
+enum fftk_store_op
+{
+    FFTK_STORE_COMPLEX  = 0,
+    FFTK_STORE_REAL     = 1, // real part only, to out0
+    FFTK_STORE_R2C_POST = 2  // half-length complex spectrum -> n+1 Hermitian bins
+};
+
+enum fftk_flags
+{
+    FFTK_F_TWIDDLE_STORE = 1 << 0, // multiply output (j, q) by W_L^{j*q}
+    FFTK_F_CHIRP_LOAD    = 1 << 1, // multiply input by conj(chirp[idx]), zero beyond blu_n
+    FFTK_F_CHIRP_STORE   = 1 << 2, // multiply output by conj(chirp[idx]), skip beyond blu_n
+    FFTK_F_CONV          = 1 << 3, // forward FFT, multiply by convb, inverse FFT
+    FFTK_F_SCALE         = 1 << 4, // multiply output by scale
+    FFTK_F_CHIRP_CONJ    = 1 << 5  // use the conjugate chirp (inverse-direction Bluestein)
+};
+
+struct fftk_params
+{
+    // transform
+    uint32_t n;                      // FFT length
+    uint32_t nf;                     // number of passes
+    uint32_t radix[FFTK_MAX_PASSES]; // radix of each pass
+    uint32_t cum[FFTK_MAX_PASSES];   // product of the radices before the pass
+    uint32_t cshift[FFTK_MAX_PASSES]; // log2(cum) when cum is a power of two, else 0xff
+    uint32_t twoff[FFTK_MAX_PASSES]; // offset of the pass in the stacked twiddle table
+    // work split
+    uint32_t T;        // threads per transform
+    uint32_t W;        // transforms per workgroup (power of two)
+    uint32_t wshift;   // log2(W)
+    uint32_t pitch;    // LDS elements between transforms of a tile
+    uint32_t padshift; // LDS index i is stored at i + (i >> padshift)
+    uint32_t wfast;    // compute phase: 1 = neighbouring lanes take neighbouring transforms
+    uint32_t nthreads;
+    uint32_t flags;
+    int32_t  dir; // -1 forward, +1 inverse
+    uint32_t load_op, store_op;
+    uint32_t n_in;  // input elements j >= n_in read as zero
+    uint32_t n_out; // output elements j >= n_out are not written
+    uint32_t in_fast_tile, out_fast_tile; // global access runs fastest along the tile dimension
+    // index space: transform, tile dimension, three outer dimensions; strides in scalars
+    uint32_t tile_cnt;
+    uint32_t oc[3];
+    int64_t  t_is, t_os, w_is, w_os, o_is[3], o_os[3];
+    // buffers (filled in at execute)
+    const void* in0;
+    const void* in1;
+    void*       out0;
+    void*       out1;
+    // tables
+    const void* tw;        // stacked per-pass twiddles
+    const void* ltw;       // two-level table for W_L^u: lo[0 .. 1<<ltw_shift), then hi[]
+    uint32_t    ltw_shift; //
+    uint32_t    aux_dim;   // which index is q: 0 none, 1 tile, 2/3/4 outer 0/1/2
+    const void* half_tw;   // e^{-2 pi i j/(2n)}, j in [0, n/2], for the real pre/post steps
+    const void* chirp;     // Bluestein chirp e^{+i pi m^2/N}, m in [0, blu_n)
+    uint32_t    blu_n;
+    uint32_t    chirp_js, chirp_qs; // logical sample index = j*chirp_js + q*chirp_qs
+    const void* convb;              // spectrum the tile is multiplied with in CONV mode
+    uint32_t    convb_qs;           // its index = j + q*convb_qs
+    double      scale;
+};
+
+// standalone even-length real post-/pre-processing over natural-order rows
+struct fftk_real_params
+{
+    uint32_t    half; // complex length L (the real length is 2L)
+    uint32_t    rows0, rows1, rows2; // three row dimensions
+    int64_t     z_s, z_r0, z_r1, z_r2; // complex side: element stride and row strides, in scalars
+    int64_t     h_s, h_r0, h_r1, h_r2; // Hermitian side
+    const void* z0;
+    const void* z1;
+    void*       zo0;
+    void*       zo1;
+    const void* h0;
+    const void* h1;
+    void*       ho0;
+    void*       ho1;
+    const void* half_tw; // e^{-2 pi i j/(2L)}, j in [0, L/2]
+    double      scale;
+    uint32_t    use_scale;
+};
+
+#endif

@@ -1,0 +1,1481 @@
+// plan.cpp -- planner, table builders and executor (host only, no HIP types).
+#include "plan.h"
+#include "gpu_rt.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <sstream>
+#include <stdexcept>
+
+namespace fftamd
+{
+
+// ---------------------------------------------------------------------------
+// limits of the tile kernel on gfx950
+
+static const size_t   LDS_SOFT_BYTES = 64 * 1024;  // preferred tile footprint (two workgroups per CU)
+static const size_t   LDS_HARD_BYTES = 160 * 1024; // LDS of one CU
+static const size_t   LDS_COL_BYTES  = 80 * 1024;  // a column tile may grow to this to keep its rows wide
+static const uint32_t MAX_THREADS    = 512;
+static const uint32_t PADSHIFT       = 4;
+// a strided ("column") pass wants at least this many bytes contiguous per row of its tile
+static const size_t   COL_RUN_BYTES  = 128;
+
+struct PlanError : std::runtime_error
+{
+    rocfft_status status;
+    PlanError(rocfft_status s, const std::string& what)
+        : std::runtime_error(what)
+        , status(s)
+    {
+    }
+};
+
+static void fail(const std::string& what)
+{
+    throw PlanError(rocfft_status_failure, what);
+}
+
+// ---------------------------------------------------------------------------
+// tables (computed in long double on the host, narrowed to the plan precision;
+// the reference computes its tables in double on the device:
+// library/src/rtc_twiddle_gen.cpp:103-188, library/src/rtc_chirp_gen.cpp:51-82)
+
+DeviceTable::~DeviceTable()
+{
+    if(dptr)
+        fftrt_free(dptr);
+}
+
+static const long double PI_L = 3.141592653589793238462643383279502884L;
+
+static void unit_root(uint64_t num, uint64_t den, long double& c, long double& s)
+{
+    // e^{-2 pi i num/den}; reduce to the first octant so cos/sin see small arguments
+    num %= den;
+    // exact symmetries keep tables bit-symmetric: handle multiples of den/8 exactly
+    long double a = 2.0L * PI_L * (long double)num / (long double)den;
+    c             = cosl(a);
+    s             = -sinl(a);
+    if(num == 0)
+    {
+        c = 1;
+        s = 0;
+    }
+    else if(4 * num == den)
+    {
+        c = 0;
+        s = -1;
+    }
+    else if(2 * num == den)
+    {
+        c = -1;
+        s = 0;
+    }
+    else if(4 * num == 3 * den)
+    {
+        c = 0;
+        s = 1;
+    }
+}
+
+struct HostTable
+{
+    std::vector<long double> v; // (re, im) pairs
+    void                     push(long double c, long double s)
+    {
+        v.push_back(c);
+        v.push_back(s);
+    }
+};
+
+static std::mutex                                   g_cache_mutex;
+static std::map<std::string, std::weak_ptr<DeviceTable>> g_cache;
+
+void table_cache_clear()
+{
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for(auto it = g_cache.begin(); it != g_cache.end();)
+    {
+        if(it->second.expired())
+            it = g_cache.erase(it);
+        else
+            ++it;
+    }
+}
+
+static TablePtr upload_table(const HostTable& h, int precision, bool dry)
+{
+    TablePtr t(new DeviceTable);
+    size_t   count = h.v.size();
+    t->bytes       = count * (precision ? sizeof(double) : sizeof(float));
+    if(dry || count == 0)
+        return t;
+    if(fftrt_malloc(&t->dptr, t->bytes) != 0)
+        fail("device allocation of a table failed");
+    int rc;
+    if(precision)
+    {
+        std::vector<double> d(count);
+        for(size_t i = 0; i < count; ++i)
+            d[i] = (double)h.v[i];
+        rc = fftrt_upload(t->dptr, d.data(), t->bytes);
+    }
+    else
+    {
+        std::vector<float> d(count);
+        for(size_t i = 0; i < count; ++i)
+            d[i] = (float)h.v[i];
+        rc = fftrt_upload(t->dptr, d.data(), t->bytes);
+    }
+    if(rc != 0)
+        fail("upload of a table failed");
+    return t;
+}
+
+template <typename Gen>
+static TablePtr cached_table(const std::string& key, int precision, bool dry, Gen gen)
+{
+    int dev = 0;
+    if(!dry)
+        fftrt_device_info(&dev, nullptr, nullptr, nullptr, 0);
+    std::ostringstream k;
+    k << key << "/p" << precision << "/d" << dev << (dry ? "/dry" : "");
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto                        it = g_cache.find(k.str());
+    if(it != g_cache.end())
+        if(TablePtr t = it->second.lock())
+            return t;
+    HostTable h;
+    gen(h);
+    TablePtr t       = upload_table(h, precision, dry);
+    g_cache[k.str()] = t;
+    return t;
+}
+
+// stacked per-pass twiddles: pass p (radix w, cumulative height c) holds
+// e^{-2 pi i jk/(c w)} at off_p + (k-1)*c + j
+static TablePtr stacked_twiddles(const std::vector<uint32_t>& radix, int precision, bool dry,
+                                 uint32_t* twoff)
+{
+    std::ostringstream key;
+    key << "stk";
+    for(uint32_t r : radix)
+        key << "_" << r;
+    uint32_t off = 0, c = 1;
+    for(size_t p = 0; p < radix.size(); ++p)
+    {
+        twoff[p] = off;
+        if(p > 0)
+            off += c * (radix[p] - 1);
+        c *= radix[p];
+    }
+    return cached_table(key.str(), precision, dry, [&](HostTable& h) {
+        uint32_t cc = 1;
+        for(size_t p = 0; p < radix.size(); ++p)
+        {
+            uint32_t w = radix[p];
+            if(p > 0)
+                for(uint32_t k = 1; k < w; ++k)
+                    for(uint32_t j = 0; j < cc; ++j)
+                    {
+                        long double co, si;
+                        unit_root((uint64_t)j * k, (uint64_t)cc * w, co, si);
+                        h.push(co, si);
+                    }
+            cc *= w;
+        }
+        if(h.v.empty())
+            h.push(1, 0);
+    });
+}
+
+// two-level table for W_L^u = lo[u & mask] * hi[u >> shift]
+static uint32_t large_twiddle_shift(uint64_t L)
+{
+    uint32_t bits = 0;
+    while(((uint64_t)1 << bits) < L)
+        ++bits;
+    return (bits + 1) / 2;
+}
+
+static TablePtr large_twiddles(uint64_t L, int precision, bool dry)
+{
+    std::ostringstream key;
+    key << "ltw_" << L;
+    return cached_table(key.str(), precision, dry, [&](HostTable& h) {
+        uint32_t shift = large_twiddle_shift(L);
+        uint64_t lo    = (uint64_t)1 << shift;
+        uint64_t hi    = (L + lo - 1) / lo + 1;
+        for(uint64_t j = 0; j < lo; ++j)
+        {
+            long double c, s;
+            unit_root(j, L, c, s);
+            h.push(c, s);
+        }
+        for(uint64_t j = 0; j < hi; ++j)
+        {
+            long double c, s;
+            unit_root((j << shift) % L, L, c, s);
+            h.push(c, s);
+        }
+    });
+}
+
+// e^{-2 pi i j/(2 half)}, j in [0, half/2]
+static TablePtr half_twiddles(uint64_t half, int precision, bool dry)
+{
+    std::ostringstream key;
+    key << "half_" << half;
+    return cached_table(key.str(), precision, dry, [&](HostTable& h) {
+        for(uint64_t j = 0; j <= half / 2; ++j)
+        {
+            long double c, s;
+            unit_root(j, 2 * half, c, s);
+            h.push(c, s);
+        }
+    });
+}
+
+static void chirp_value(uint64_t m, uint64_t N, long double& c, long double& s)
+{
+    // e^{+i pi m^2/N} with m^2 reduced mod 2N exactly
+    unsigned __int128 sq = (unsigned __int128)m * m;
+    uint64_t          u  = (uint64_t)(sq % (2 * (unsigned __int128)N));
+    unit_root(u, 2 * N, c, s);
+    s = -s;
+}
+
+static TablePtr chirp_table(uint64_t N, int precision, bool dry)
+{
+    std::ostringstream key;
+    key << "chirp_" << N;
+    return cached_table(key.str(), precision, dry, [&](HostTable& h) {
+        for(uint64_t m = 0; m < N; ++m)
+        {
+            long double c, s;
+            chirp_value(m, N, c, s);
+            h.push(c, s);
+        }
+    });
+}
+
+// ---------------------------------------------------------------------------
+// factorisation
+
+static bool factorize(uint64_t n, std::vector<uint32_t>& radix)
+{
+    radix.clear();
+    if(n <= 1)
+        return n == 1;
+    static const uint32_t odd[] = {13, 11, 7, 5, 3};
+    uint64_t              m     = n;
+    for(uint32_t r : odd)
+        while(m % r == 0)
+        {
+            radix.push_back(r);
+            m /= r;
+        }
+    uint32_t k = 0;
+    while(m % 2 == 0)
+    {
+        ++k;
+        m /= 2;
+    }
+    if(m != 1)
+        return false;
+    // 2^k as radix-16 passes plus one or two smaller ones
+    uint32_t a = k / 4, b = k % 4;
+    std::vector<uint32_t> two;
+    if(b == 1 && a >= 1)
+    {
+        --a;
+        two.push_back(8);
+        two.push_back(4);
+    }
+    else if(b == 1)
+        two.push_back(2);
+    else if(b == 2)
+        two.push_back(4);
+    else if(b == 3)
+        two.push_back(8);
+    for(uint32_t i = 0; i < a; ++i)
+        radix.push_back(16);
+    for(uint32_t r : two)
+        radix.push_back(r);
+    return radix.size() <= FFTK_MAX_PASSES;
+}
+
+static uint32_t threads_per_transform(uint64_t n, const std::vector<uint32_t>& radix)
+{
+    uint32_t T = 1;
+    for(uint32_t r : radix)
+    {
+        uint32_t m     = (uint32_t)(n / r);
+        uint32_t slots = FFTK_REG_ELEMS / r;
+        T              = std::max(T, (m + slots - 1) / slots);
+    }
+    return T;
+}
+
+static uint32_t lds_pitch(uint32_t n)
+{
+    uint32_t p = n + ((n - 1) >> PADSHIFT) + 1;
+    return p | 1u; // odd, so neighbouring transforms start in different banks
+}
+
+// can a single tile kernel transform length n (one transform per workgroup at least)?
+static bool single_kernel_length(uint64_t n, size_t elem_bytes)
+{
+    if(n < 1 || n > 65536)
+        return false;
+    std::vector<uint32_t> radix;
+    if(!factorize(n, radix))
+        return false;
+    if(threads_per_transform(n, radix) > MAX_THREADS)
+        return false;
+    return (size_t)lds_pitch((uint32_t)n) * elem_bytes <= LDS_HARD_BYTES;
+}
+
+// longest length a strided pass handles while keeping COL_RUN_BYTES contiguous per row
+static bool column_kernel_length(uint64_t n, size_t elem_bytes)
+{
+    if(!single_kernel_length(n, elem_bytes))
+        return false;
+    size_t w = std::max<size_t>(1, COL_RUN_BYTES / elem_bytes);
+    return (size_t)lds_pitch((uint32_t)n) * elem_bytes * w <= LDS_COL_BYTES;
+}
+
+static uint32_t floor_pow2(uint64_t v)
+{
+    uint32_t p = 1;
+    while((uint64_t)p * 2 <= v)
+        p *= 2;
+    return p;
+}
+static uint32_t ceil_pow2(uint64_t v)
+{
+    uint32_t p = 1;
+    while(p < v)
+        p *= 2;
+    return p;
+}
+static uint32_t log2u(uint32_t v)
+{
+    uint32_t s = 0;
+    while((1u << s) < v)
+        ++s;
+    return s;
+}
+
+// ---------------------------------------------------------------------------
+// views: a logical array with up to three dimensions plus batch, strides in scalars
+
+struct View
+{
+    IoRef   io;
+    int64_t stride[4] = {0, 0, 0, 0};
+};
+
+static View complex_view(int buf, rocfft_array_type type, const size_t* stride, size_t dist,
+                         const size_t* offset, size_t rank)
+{
+    View v;
+    v.io.buf    = buf;
+    bool planar = type == rocfft_array_type_complex_planar || type == rocfft_array_type_hermitian_planar;
+    v.io.planar = planar;
+    int64_t m   = planar ? 1 : 2;
+    v.io.im_delta = 1;
+    v.io.off0     = m * (int64_t)offset[0];
+    v.io.off1     = planar ? (int64_t)offset[1] : 0;
+    for(size_t d = 0; d < 3; ++d)
+        v.stride[d] = d < rank ? m * (int64_t)stride[d] : 0;
+    v.stride[3] = m * (int64_t)dist;
+    return v;
+}
+
+// real array seen as complex pairs along dimension 0 (even-length real transforms)
+static View realpair_view(int buf, const size_t* stride, size_t dist, const size_t* offset,
+                          size_t rank)
+{
+    View v;
+    v.io.buf      = buf;
+    v.io.planar   = false;
+    v.io.im_delta = (int64_t)stride[0];
+    v.io.off0     = (int64_t)offset[0];
+    for(size_t d = 0; d < 3; ++d)
+        v.stride[d] = d < rank ? (int64_t)stride[d] : 0;
+    v.stride[0] *= 2;
+    v.stride[3] = (int64_t)dist;
+    return v;
+}
+
+// real array, one scalar per element
+static View real_view(int buf, const size_t* stride, size_t dist, const size_t* offset, size_t rank)
+{
+    View v;
+    v.io.buf      = buf;
+    v.io.planar   = false;
+    v.io.im_delta = 0;
+    v.io.off0     = (int64_t)offset[0];
+    for(size_t d = 0; d < 3; ++d)
+        v.stride[d] = d < rank ? (int64_t)stride[d] : 0;
+    v.stride[3] = (int64_t)dist;
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// tile pass construction
+
+struct Axis
+{
+    uint32_t cnt;
+    int64_t  is, os;
+    bool     aux;
+};
+
+struct TileSpec
+{
+    uint32_t          n        = 1;
+    int64_t           t_is = 0, t_os = 0;
+    std::vector<Axis> others;
+    IoRef             src, dst;
+    int64_t           src_extra = 0, dst_extra = 0; // extra scalar offsets
+    uint32_t          load_op = FFTK_LOAD_COMPLEX, store_op = FFTK_STORE_COMPLEX;
+    uint32_t          flags = 0;
+    int               dir   = -1;
+    uint32_t          n_in = 0, n_out = 0; // 0 = n
+    TablePtr          ltw, half_tw, chirp, convb;
+    uint32_t          ltw_shift = 0;
+    uint32_t          blu_n = 0, chirp_js = 0, chirp_qs = 0, convb_qs = 0;
+    double            scale = 1.0;
+    std::string       note;
+    bool              src_real_scalar = false, dst_real_scalar = false;
+};
+
+static bool io_vec_ok(const IoRef& io, bool real_scalar)
+{
+    return !io.planar && !real_scalar && io.im_delta == 1 && (io.off0 % 2 == 0);
+}
+
+static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
+{
+    const size_t esize = precision ? 16 : 8;
+    PassRec      rec;
+    rec.kind = PASS_TILE;
+    rec.src  = s.src;
+    rec.dst  = s.dst;
+    rec.src.off0 += s.src_extra;
+    rec.src.off1 += s.src_extra;
+    rec.dst.off0 += s.dst_extra;
+    rec.dst.off1 += s.dst_extra;
+    rec.note = s.note;
+
+    fftk_params& k = rec.kp;
+    memset(&k, 0, sizeof(k));
+    k.n = s.n;
+    std::vector<uint32_t> radix;
+    if(!factorize(s.n, radix))
+        fail("length has no kernel factorisation");
+    k.nf         = (uint32_t)radix.size();
+    uint32_t cum = 1;
+    for(size_t p = 0; p < radix.size(); ++p)
+    {
+        k.radix[p]  = radix[p];
+        k.cum[p]    = cum;
+        k.cshift[p] = (cum & (cum - 1)) == 0 ? log2u(cum) : 0xff;
+        cum *= radix[p];
+    }
+    TablePtr tw = stacked_twiddles(radix, precision, dry, k.twoff);
+    k.tw        = tw->dptr;
+    rec.tables.push_back(tw);
+
+    // drop unit axes, merge axes that continue one another
+    std::vector<Axis> ax;
+    for(const Axis& a : s.others)
+        if(a.cnt > 1 || a.aux)
+            ax.push_back(a);
+    for(bool merged = true; merged;)
+    {
+        merged = false;
+        for(size_t i = 0; i < ax.size() && !merged; ++i)
+            for(size_t j = 0; j < ax.size() && !merged; ++j)
+            {
+                if(i == j || ax[i].aux || ax[j].aux)
+                    continue;
+                if(ax[i].is * (int64_t)ax[i].cnt == ax[j].is && ax[i].os * (int64_t)ax[i].cnt == ax[j].os
+                   && (uint64_t)ax[i].cnt * ax[j].cnt < (1ull << 31))
+                {
+                    ax[i].cnt *= ax[j].cnt;
+                    ax.erase(ax.begin() + (long)j);
+                    merged = true;
+                }
+            }
+    }
+    if(ax.size() > 4)
+        fail("too many independent dimensions for one pass");
+
+    // tile axis: the one global accesses should run along when the transform axis is strided
+    int     tile = -1;
+    int64_t best = 0;
+    auto    pick = [&](bool by_in) {
+        for(size_t i = 0; i < ax.size(); ++i)
+        {
+            int64_t st = by_in ? ax[i].is : ax[i].os;
+            if(tile < 0 || st < best)
+            {
+                tile = (int)i;
+                best = st;
+            }
+        }
+    };
+    bool row_in = true, row_out = true;
+    for(const Axis& a : ax)
+    {
+        if(a.cnt > 1 && a.is < s.t_is)
+            row_in = false;
+        if(a.cnt > 1 && a.os < s.t_os)
+            row_out = false;
+    }
+    if(!ax.empty())
+    {
+        if(!row_in)
+            pick(true);
+        else if(!row_out)
+            pick(false);
+        else
+            pick(true);
+    }
+    Axis tile_axis = {1, 0, 0, false};
+    if(tile >= 0)
+    {
+        tile_axis = ax[(size_t)tile];
+        ax.erase(ax.begin() + tile);
+    }
+    if(ax.size() > 3)
+        fail("too many independent dimensions for one pass");
+    k.tile_cnt      = tile_axis.cnt;
+    k.w_is          = tile_axis.is;
+    k.w_os          = tile_axis.os;
+    k.t_is          = s.t_is;
+    k.t_os          = s.t_os;
+    k.in_fast_tile  = (tile_axis.cnt > 1 && tile_axis.is < s.t_is) ? 1 : 0;
+    k.out_fast_tile = (tile_axis.cnt > 1 && tile_axis.os < s.t_os) ? 1 : 0;
+    k.aux_dim       = tile_axis.aux ? 1 : 0;
+    for(int i = 0; i < 3; ++i)
+    {
+        k.oc[i]   = 1;
+        k.o_is[i] = k.o_os[i] = 0;
+    }
+    for(size_t i = 0; i < ax.size(); ++i)
+    {
+        k.oc[i]   = ax[i].cnt;
+        k.o_is[i] = ax[i].is;
+        k.o_os[i] = ax[i].os;
+        if(ax[i].aux)
+            k.aux_dim = 2 + (uint32_t)i;
+    }
+
+    // work split
+    k.T        = threads_per_transform(s.n, radix);
+    k.padshift = PADSHIFT;
+    k.pitch    = lds_pitch(s.n);
+    if(k.T > MAX_THREADS)
+        fail("transform too long for one workgroup");
+    size_t   per_tile  = (size_t)k.pitch * esize;
+    uint32_t w_threads = floor_pow2(MAX_THREADS / k.T);
+    uint32_t w_lds     = per_tile <= LDS_SOFT_BYTES ? floor_pow2(LDS_SOFT_BYTES / per_tile) : 1;
+    if(per_tile > LDS_HARD_BYTES)
+        fail("transform too long for the LDS of one compute unit");
+    uint32_t w_cap  = ceil_pow2(k.tile_cnt);
+    bool     column = k.in_fast_tile || k.out_fast_tile;
+    uint32_t W;
+    if(column)
+    {
+        // keep COL_RUN_BYTES contiguous per tile row even if that costs occupancy
+        uint32_t w_run = (uint32_t)std::max<size_t>(1, COL_RUN_BYTES / esize);
+        if(w_lds < w_run && per_tile * w_run <= LDS_COL_BYTES)
+            w_lds = w_run;
+        W = std::min(std::min<uint32_t>(64, w_threads), std::min(w_lds, w_cap));
+    }
+    else
+    {
+        uint32_t target = floor_pow2(std::max<uint32_t>(1, 256 / k.T));
+        W               = std::min(std::min(target, w_threads), std::min(w_lds, w_cap));
+    }
+    W          = std::max<uint32_t>(W, 1);
+    k.W        = W;
+    k.wshift   = log2u(W);
+    k.wfast    = W >= 16 ? 1 : 0;
+    k.nthreads = (k.T * W + 63) / 64 * 64;
+    rec.lds    = (size_t)k.pitch * W * esize;
+    uint64_t ntile = (k.tile_cnt + W - 1) / W;
+    uint64_t grid  = ntile * k.oc[0] * k.oc[1] * k.oc[2];
+    if(grid == 0 || grid >= (1ull << 31))
+        fail("grid too large");
+    rec.grid = (uint32_t)grid;
+
+    k.flags    = s.flags;
+    k.dir      = s.dir;
+    k.load_op  = s.load_op;
+    k.store_op = s.store_op;
+    k.n_in     = s.n_in ? s.n_in : s.n;
+    k.n_out    = s.n_out ? s.n_out : s.n;
+    if(s.ltw)
+    {
+        k.ltw       = s.ltw->dptr;
+        k.ltw_shift = s.ltw_shift;
+        rec.tables.push_back(s.ltw);
+    }
+    if(s.half_tw)
+    {
+        k.half_tw = s.half_tw->dptr;
+        rec.tables.push_back(s.half_tw);
+    }
+    if(s.chirp)
+    {
+        k.chirp    = s.chirp->dptr;
+        k.blu_n    = s.blu_n;
+        k.chirp_js = s.chirp_js;
+        k.chirp_qs = s.chirp_qs;
+        rec.tables.push_back(s.chirp);
+    }
+    if(s.convb)
+    {
+        k.convb    = s.convb->dptr;
+        k.convb_qs = s.convb_qs;
+        rec.tables.push_back(s.convb);
+    }
+    k.scale = s.scale;
+
+    // one access per (re, im) pair needs interleaved data with even scalar strides
+    bool vec = io_vec_ok(rec.src, s.src_real_scalar) && io_vec_ok(rec.dst, s.dst_real_scalar);
+    auto even = [](int64_t v) { return v % 2 == 0; };
+    vec = vec && even(k.t_is) && even(k.t_os) && even(k.w_is) && even(k.w_os);
+    for(int i = 0; i < 3; ++i)
+        vec = vec && even(k.o_is[i]) && even(k.o_os[i]);
+    if(s.load_op == FFTK_LOAD_REAL || s.store_op == FFTK_STORE_REAL)
+        vec = false;
+    rec.vec_ok = vec;
+    return rec;
+}
+
+// ---------------------------------------------------------------------------
+// emitters
+
+struct Builder
+{
+    ExecPlan* plan;
+    int       precision;
+    bool      dry;
+    size_t    esize;
+    void      need_tmp(size_t elems)
+    {
+        plan->tmp_elems = std::max(plan->tmp_elems, elems);
+    }
+    void need_blu(size_t elems)
+    {
+        plan->blu_elems = std::max(plan->blu_elems, elems);
+    }
+};
+
+struct Other
+{
+    uint32_t cnt;
+    int64_t  is, os;
+};
+
+struct DimOps
+{
+    // fused input/output operations of the first/last pass of the dimension
+    uint32_t load_op  = FFTK_LOAD_COMPLEX;
+    uint32_t store_op = FFTK_STORE_COMPLEX;
+    uint32_t n_in     = 0; // logical input length (0 = n)
+    uint32_t n_out    = 0; // outputs kept (0 = n)
+    bool     src_real_scalar = false, dst_real_scalar = false;
+    TablePtr half_tw;
+    double   scale     = 1.0;
+    bool     has_scale = false;
+};
+
+static std::string dims_note(const char* what, uint64_t n)
+{
+    std::ostringstream o;
+    o << what << " n=" << n;
+    return o.str();
+}
+
+static void split_length(uint64_t n, size_t esize, bool column, uint64_t& n1, uint64_t& n0)
+{
+    // n = n1 * n0, both single-kernel lengths, as balanced as possible; n0 is the
+    // length of the pass that reads rows of the intermediate array
+    uint64_t best = 0;
+    double   root = std::sqrt((double)n);
+    for(uint64_t a = 2; a * a <= n; ++a)
+    {
+        if(n % a)
+            continue;
+        uint64_t b  = n / a;
+        auto     ok = [&](uint64_t v) {
+            return column ? column_kernel_length(v, esize) : single_kernel_length(v, esize);
+        };
+        if(!ok(a) || !ok(b))
+            continue;
+        if(best == 0 || std::fabs((double)a - root) < std::fabs((double)best - root))
+            best = a;
+    }
+    if(best == 0)
+    {
+        n1 = n0 = 0;
+        return;
+    }
+    n1 = best;
+    n0 = n / best;
+}
+
+static bool smooth(uint64_t n)
+{
+    std::vector<uint32_t> r;
+    for(uint32_t p : {2u, 3u, 5u, 7u, 11u, 13u})
+        while(n % p == 0)
+            n /= p;
+    return n == 1;
+}
+
+static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t M1, uint64_t M0,
+                                   bool conj_chirp);
+
+// One dimension of complex transforms: length n along an axis with scalar strides
+// (t_is, t_os); `others` are the remaining index dimensions.  src and dst may be
+// the same buffer: every decomposition below finishes reading src before dst is
+// written, going through the work buffer where a pass cannot run in place.
+static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const std::vector<Other>& others,
+                     const IoRef& src, const IoRef& dst, int dir, const DimOps& ops)
+{
+    const size_t esize = b.esize;
+    uint64_t     lines = 1;
+    for(const Other& o : others)
+        lines *= o.cnt;
+
+    // is the transform axis the fastest one on both sides?
+    bool column = false;
+    for(const Other& o : others)
+        if(o.cnt > 1 && (o.is < t_is || o.os < t_os))
+            column = true;
+    bool plain = ops.load_op == FFTK_LOAD_COMPLEX && ops.store_op == FFTK_STORE_COMPLEX && !ops.n_in
+                 && !ops.n_out;
+
+    auto base_spec = [&]() {
+        TileSpec s;
+        s.dir = dir;
+        return s;
+    };
+    auto add_others = [&](TileSpec& s, bool in_user, bool out_user, const std::vector<int64_t>& packed) {
+        for(size_t i = 0; i < others.size(); ++i)
+            s.others.push_back({others[i].cnt, in_user ? others[i].is : packed[i],
+                                out_user ? others[i].os : packed[i], false});
+    };
+    // strides of the `others` axes in a packed scratch array of line length `linelen` complex
+    auto packed_strides = [&](uint64_t linelen) {
+        std::vector<int64_t> p;
+        int64_t              st = 2 * (int64_t)linelen;
+        for(const Other& o : others)
+        {
+            p.push_back(st);
+            st *= o.cnt;
+        }
+        return p;
+    };
+    IoRef tmp;
+    tmp.buf = BUF_TMP;
+    IoRef blu;
+    blu.buf = BUF_BLU;
+
+    bool single = column ? (column_kernel_length(n, esize) || !plain) && single_kernel_length(n, esize)
+                         : single_kernel_length(n, esize);
+    // a strided pass that is not "plain" (fused real/odd handling) stays single if it fits at all
+    if(single)
+    {
+        TileSpec s = base_spec();
+        s.n        = (uint32_t)n;
+        s.t_is     = t_is;
+        s.t_os     = t_os;
+        s.src      = src;
+        s.dst      = dst;
+        add_others(s, true, true, {});
+        s.load_op         = ops.load_op;
+        s.store_op        = ops.store_op;
+        s.n_in            = ops.n_in;
+        s.n_out           = ops.n_out;
+        s.half_tw         = ops.half_tw;
+        s.src_real_scalar = ops.src_real_scalar;
+        s.dst_real_scalar = ops.dst_real_scalar;
+        if(ops.has_scale)
+        {
+            s.flags |= FFTK_F_SCALE;
+            s.scale = ops.scale;
+        }
+        s.note = dims_note(column ? "column fft" : "row fft", n);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        return;
+    }
+
+    if(smooth(n))
+    {
+        if(!plain)
+            fail("this real-transform length needs a decomposition that is not implemented");
+        uint64_t n1, n0;
+        split_length(n, esize, column, n1, n0);
+        if(n1 == 0)
+            split_length(n, esize, false, n1, n0);
+        if(n1 == 0)
+            fail("length too large for a two-pass decomposition");
+        // pass A: for every n0' an n1-point FFT over the stride-n0 samples, times W_n^{k1 n0'},
+        // written to scratch at [line][k1*n0 + n0']
+        // pass B: for every k1 an n0-point FFT over n0', written to dst at k0*n1 + k1
+        // (the reference's two-kernel large 1D, library/src/tree_node_1D.cpp:404-469)
+        b.need_tmp(lines * n);
+        std::vector<int64_t> pk = packed_strides(n);
+        TablePtr             ltw = large_twiddles(n, b.precision, b.dry);
+        {
+            TileSpec s = base_spec();
+            s.n        = (uint32_t)n1;
+            s.t_is     = (int64_t)n0 * t_is;
+            s.t_os     = (int64_t)n0 * 2;
+            s.src      = src;
+            s.dst      = tmp;
+            s.others.push_back({(uint32_t)n0, t_is, 2, true});
+            add_others(s, true, false, pk);
+            s.flags |= FFTK_F_TWIDDLE_STORE;
+            s.ltw       = ltw;
+            s.ltw_shift = large_twiddle_shift(n);
+            s.note      = dims_note("split A (column fft + twiddle)", n1);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        {
+            TileSpec s = base_spec();
+            s.n        = (uint32_t)n0;
+            s.t_is     = 2;
+            s.t_os     = (int64_t)n1 * t_os;
+            s.src      = tmp;
+            s.dst      = dst;
+            s.others.push_back({(uint32_t)n1, (int64_t)n0 * 2, t_os, false});
+            add_others(s, false, true, pk);
+            if(ops.has_scale)
+            {
+                s.flags |= FFTK_F_SCALE;
+                s.scale = ops.scale;
+            }
+            s.note = dims_note("split B (row fft, transposed store)", n0);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        return;
+    }
+
+    // Bluestein chirp-z (reference: library/src/tree_node_bluestein.cpp:27-285,
+    // library/src/rtc_bluestein_gen.cpp:170-380).  The convolution length M is the
+    // next power of two >= 2n-1; chirp and its spectrum are plan-time tables.
+    if(ops.store_op != FFTK_STORE_COMPLEX && ops.store_op != FFTK_STORE_REAL)
+        fail("Bluestein cannot be combined with this real-transform step");
+    if(ops.load_op == FFTK_LOAD_C2R_PRE)
+        fail("Bluestein cannot be combined with this real-transform step");
+    uint64_t N = n;
+    uint64_t M = ceil_pow2(2 * N - 1);
+    if(M >= (1ull << 31))
+        fail("length too large");
+    bool     conj_chirp = dir > 0;
+    TablePtr chirp      = chirp_table(N, b.precision, b.dry);
+    double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
+    uint32_t cflag      = conj_chirp ? FFTK_F_CHIRP_CONJ : 0;
+    // the whole convolution in one workgroup when M fits; strided data must keep a wide tile
+    bool one = column ? column_kernel_length(M, esize) : single_kernel_length(M, esize);
+    if(!one && column && single_kernel_length(M, esize) && M <= 4096)
+        one = true;
+    if(one)
+    {
+        TablePtr bs = bluestein_spectrum(b, N, M, 0, 0, conj_chirp);
+        TileSpec s  = base_spec();
+        s.dir       = -1;
+        s.n         = (uint32_t)M;
+        s.t_is      = t_is;
+        s.t_os      = t_os;
+        s.src       = src;
+        s.dst       = dst;
+        add_others(s, true, true, {});
+        s.load_op         = ops.load_op;
+        s.store_op        = ops.store_op;
+        s.src_real_scalar = ops.src_real_scalar;
+        s.dst_real_scalar = ops.dst_real_scalar;
+        s.n_in            = (uint32_t)N;
+        s.n_out           = ops.n_out ? ops.n_out : (uint32_t)N;
+        s.flags |= FFTK_F_CHIRP_LOAD | FFTK_F_CHIRP_STORE | FFTK_F_CONV | FFTK_F_SCALE | cflag;
+        s.chirp    = chirp;
+        s.blu_n    = (uint32_t)N;
+        s.chirp_js = 1;
+        s.chirp_qs = 0;
+        s.convb    = bs;
+        s.convb_qs = 0;
+        s.scale    = scale;
+        s.note     = dims_note("bluestein single kernel, M", M);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        return;
+    }
+    if(ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out)
+        fail("odd-length real transforms of this size are not implemented");
+    // M = M1*M0: rows of length M0 are transformed, multiplied and transformed back by
+    // one kernel, so that kernel gets the long factor; the strided passes get M1
+    uint64_t M0 = 4096, M1 = M / M0;
+    while(M1 > 1 && !single_kernel_length(M1, esize))
+        fail("Bluestein length too large");
+    if(M1 < 2)
+        fail("internal: Bluestein split of a short length");
+    TablePtr bs  = bluestein_spectrum(b, N, M, M1, M0, conj_chirp);
+    TablePtr ltw = large_twiddles(M, b.precision, b.dry);
+    b.need_blu(lines * M);
+    std::vector<int64_t> pk = packed_strides(M);
+    {
+        // Z1: chirp multiply + zero pad fused into the load of the column FFT over n1
+        TileSpec s = base_spec();
+        s.dir      = -1;
+        s.n        = (uint32_t)M1;
+        s.t_is     = (int64_t)M0 * t_is;
+        s.t_os     = (int64_t)M0 * 2;
+        s.src      = src;
+        s.dst      = blu;
+        s.others.push_back({(uint32_t)M0, t_is, 2, true});
+        add_others(s, true, false, pk);
+        s.load_op         = ops.load_op;
+        s.src_real_scalar = ops.src_real_scalar;
+        s.flags |= FFTK_F_CHIRP_LOAD | FFTK_F_TWIDDLE_STORE | cflag;
+        s.chirp     = chirp;
+        s.blu_n     = (uint32_t)N;
+        s.chirp_js  = (uint32_t)M0;
+        s.chirp_qs  = 1;
+        s.ltw       = ltw;
+        s.ltw_shift = large_twiddle_shift(M);
+        s.note      = dims_note("bluestein Z1 (chirp, pad, column fft, twiddle)", M1);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    }
+    {
+        // Z2: row FFT, multiply by the chirp spectrum, inverse row FFT, conjugate twiddle
+        TileSpec s = base_spec();
+        s.dir      = -1;
+        s.n        = (uint32_t)M0;
+        s.t_is = s.t_os = 2;
+        s.src = s.dst = blu;
+        s.others.push_back({(uint32_t)M1, (int64_t)M0 * 2, (int64_t)M0 * 2, true});
+        add_others(s, false, false, pk);
+        s.flags |= FFTK_F_CONV | FFTK_F_TWIDDLE_STORE;
+        s.convb     = bs;
+        s.convb_qs  = (uint32_t)M0;
+        s.ltw       = ltw;
+        s.ltw_shift = large_twiddle_shift(M);
+        s.note      = dims_note("bluestein Z2 (row fft, multiply, inverse row fft, twiddle)", M0);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    }
+    {
+        // Z3: inverse column FFT, multiply by the chirp, scale by 1/M, keep n outputs
+        TileSpec s = base_spec();
+        s.dir      = +1;
+        s.n        = (uint32_t)M1;
+        s.t_is     = (int64_t)M0 * 2;
+        s.t_os     = (int64_t)M0 * t_os;
+        s.src      = blu;
+        s.dst      = dst;
+        s.others.push_back({(uint32_t)M0, 2, t_os, true});
+        add_others(s, false, true, pk);
+        s.store_op        = ops.store_op;
+        s.dst_real_scalar = ops.dst_real_scalar;
+        s.flags |= FFTK_F_CHIRP_STORE | FFTK_F_SCALE | cflag;
+        s.chirp    = chirp;
+        s.blu_n    = (uint32_t)N;
+        s.chirp_js = (uint32_t)M0;
+        s.chirp_qs = 1;
+        s.scale    = scale;
+        s.note     = dims_note("bluestein Z3 (inverse column fft, chirp, scale)", M1);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    }
+}
+
+// FFT_M of the wrapped chirp, computed on the GPU in double precision with this
+// library's own passes and narrowed to the plan precision.  For a split M the
+// result is kept in the order the convolution kernel meets it: [k1*M0 + k0].
+static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t M1, uint64_t M0,
+                                   bool conj_chirp)
+{
+    std::ostringstream key;
+    key << "bspec_" << N << "_" << M << "_" << M1 << "_" << M0 << (conj_chirp ? "c" : "f");
+    int dev = 0;
+    if(!b.dry)
+        fftrt_device_info(&dev, nullptr, nullptr, nullptr, 0);
+    key << "/p" << b.precision << "/d" << dev << (b.dry ? "/dry" : "");
+    {
+        std::lock_guard<std::mutex> lock(g_cache_mutex);
+        auto                        it = g_cache.find(key.str());
+        if(it != g_cache.end())
+            if(TablePtr t = it->second.lock())
+                return t;
+    }
+    TablePtr out(new DeviceTable);
+    out->bytes = M * (b.precision ? 16 : 8);
+    if(!b.dry)
+    {
+        std::vector<double> w(2 * M, 0.0);
+        for(uint64_t m = 0; m < N; ++m)
+        {
+            long double c, s;
+            chirp_value(m, N, c, s);
+            if(conj_chirp)
+                s = -s;
+            w[2 * m]     = (double)c;
+            w[2 * m + 1] = (double)s;
+            if(m)
+            {
+                w[2 * (M - m)]     = (double)c;
+                w[2 * (M - m) + 1] = (double)s;
+            }
+        }
+        void* dbuf = nullptr;
+        if(fftrt_malloc(&dbuf, 2 * M * sizeof(double)) != 0)
+            fail("device allocation failed");
+        std::shared_ptr<void> guard(dbuf, [](void* p) { fftrt_free(p); });
+        if(fftrt_upload(dbuf, w.data(), 2 * M * sizeof(double)) != 0)
+            fail("upload failed");
+        ExecPlan sub;
+        sub.precision  = 1;
+        sub.elem_bytes = 16;
+        Builder sb{&sub, 1, false, 16};
+        IoRef   io;
+        io.buf = BUF_IN;
+        DimOps none;
+        if(M1 == 0)
+            emit_dim(sb, M, 2, 2, {}, io, io, -1, none);
+        else
+        {
+            TablePtr ltw = large_twiddles(M, 1, false);
+            TileSpec a;
+            a.dir  = -1;
+            a.n    = (uint32_t)M1;
+            a.t_is = a.t_os = (int64_t)M0 * 2;
+            a.src = a.dst = io;
+            a.others.push_back({(uint32_t)M0, 2, 2, true});
+            a.flags |= FFTK_F_TWIDDLE_STORE;
+            a.ltw       = ltw;
+            a.ltw_shift = large_twiddle_shift(M);
+            sub.passes.push_back(make_tile_pass(a, 1, false));
+            TileSpec r;
+            r.dir  = -1;
+            r.n    = (uint32_t)M0;
+            r.t_is = r.t_os = 2;
+            r.src = r.dst = io;
+            r.others.push_back({(uint32_t)M1, (int64_t)M0 * 2, (int64_t)M0 * 2, false});
+            sub.passes.push_back(make_tile_pass(r, 1, false));
+        }
+        void* bufs[2] = {dbuf, nullptr};
+        if(run_exec_plan(sub, bufs, bufs, nullptr, nullptr) != rocfft_status_success)
+            fail("computing the Bluestein chirp spectrum failed");
+        if(fftrt_stream_sync(nullptr) != 0)
+            fail("computing the Bluestein chirp spectrum failed");
+        if(fftrt_download(w.data(), dbuf, 2 * M * sizeof(double)) != 0)
+            fail("download failed");
+        if(fftrt_malloc(&out->dptr, out->bytes) != 0)
+            fail("device allocation failed");
+        int rc;
+        if(b.precision)
+            rc = fftrt_upload(out->dptr, w.data(), out->bytes);
+        else
+        {
+            std::vector<float> f(2 * M);
+            for(size_t i = 0; i < 2 * M; ++i)
+                f[i] = (float)w[i];
+            rc = fftrt_upload(out->dptr, f.data(), out->bytes);
+        }
+        if(rc != 0)
+            fail("upload failed");
+    }
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    g_cache[key.str()] = out;
+    return out;
+}
+
+// standalone even-length post/pre pass over natural-order rows
+static void emit_real_step(Builder& b, PassKind kind, uint64_t half, const std::vector<Other>& rows,
+                           int64_t z_s, const IoRef& z, int64_t h_s, const IoRef& h, double scale,
+                           bool has_scale)
+{
+    // rows: is = stride on the complex (z) side, os = stride on the Hermitian (h) side
+    if(rows.size() > 3)
+        fail("too many dimensions");
+    PassRec rec;
+    rec.kind = kind;
+    memset(&rec.kp, 0, sizeof(rec.kp));
+    fftk_real_params& r = rec.rp;
+    memset(&r, 0, sizeof(r));
+    r.half  = (uint32_t)half;
+    r.rows0 = r.rows1 = r.rows2 = 1;
+    uint32_t* cnt[3]            = {&r.rows0, &r.rows1, &r.rows2};
+    int64_t*  zs[3]             = {&r.z_r0, &r.z_r1, &r.z_r2};
+    int64_t*  hs[3]             = {&r.h_r0, &r.h_r1, &r.h_r2};
+    for(size_t i = 0; i < rows.size(); ++i)
+    {
+        *cnt[i] = rows[i].cnt;
+        *zs[i]  = rows[i].is;
+        *hs[i]  = rows[i].os;
+    }
+    r.z_s         = z_s;
+    r.h_s         = h_s;
+    r.scale       = scale;
+    r.use_scale   = has_scale ? 1 : 0;
+    TablePtr tw   = half_twiddles(half, b.precision, b.dry);
+    r.half_tw     = tw->dptr;
+    rec.tables.push_back(tw);
+    if(kind == PASS_REAL_POST)
+    {
+        rec.src = z;
+        rec.dst = h;
+    }
+    else
+    {
+        rec.src = h;
+        rec.dst = z;
+    }
+    rec.note = dims_note(kind == PASS_REAL_POST ? "real post-process" : "real pre-process", 2 * half);
+    b.plan->passes.push_back(rec);
+}
+
+// ---------------------------------------------------------------------------
+// whole transforms
+
+static std::vector<Other> other_axes(const View& in, const View& out, const size_t* len, size_t rank,
+                                     size_t batch, size_t skip)
+{
+    std::vector<Other> o;
+    for(size_t d = 0; d < rank; ++d)
+        if(d != skip)
+            o.push_back({(uint32_t)len[d], in.stride[d], out.stride[d]});
+    o.push_back({(uint32_t)batch, in.stride[3], out.stride[3]});
+    return o;
+}
+
+static void check_sizes(const Problem& p)
+{
+    for(size_t d = 0; d < p.rank; ++d)
+        if(p.len[d] == 0 || p.len[d] >= (1ull << 31))
+            throw PlanError(rocfft_status_invalid_dimensions, "bad length");
+    if(p.batch == 0 || p.batch >= (1ull << 31))
+        throw PlanError(rocfft_status_failure, "bad batch");
+}
+
+rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::string& err)
+{
+    try
+    {
+        if(p.precision != rocfft_precision_single && p.precision != rocfft_precision_double)
+            fail("half precision is not implemented");
+        check_sizes(p);
+        plan.passes.clear();
+        plan.precision  = p.precision == rocfft_precision_double ? 1 : 0;
+        plan.elem_bytes = plan.precision ? 16 : 8;
+        plan.inplace    = p.placement == rocfft_placement_inplace;
+        Builder b{&plan, plan.precision, dry, plan.elem_bytes};
+        const int out_buf = plan.inplace ? BUF_IN : BUF_OUT;
+
+        const bool is_real = p.type == rocfft_transform_type_real_forward
+                             || p.type == rocfft_transform_type_real_inverse;
+        DimOps scale_ops;
+        scale_ops.scale     = p.scale;
+        scale_ops.has_scale = p.has_scale;
+
+        if(!is_real)
+        {
+            int  dir = p.type == rocfft_transform_type_complex_forward ? -1 : +1;
+            View in  = complex_view(BUF_IN, p.in_type, p.istride, p.idist, p.ioffset, p.rank);
+            View out = complex_view(out_buf, p.out_type, p.ostride, p.odist, p.ooffset, p.rank);
+            if(plan.inplace)
+                for(int d = 0; d < 4; ++d)
+                    if(in.stride[d] != out.stride[d] && (d == 3 || (size_t)d < p.rank))
+                        fail("in-place transforms need identical input and output layouts");
+            for(size_t d = 0; d < p.rank; ++d)
+            {
+                const View& src = d == 0 ? in : out;
+                DimOps      ops = d + 1 == p.rank ? scale_ops : DimOps();
+                emit_dim(b, p.len[d], src.stride[d], out.stride[d],
+                         other_axes(src, out, p.len, p.rank, p.batch, d), src.io, out.io, dir, ops);
+            }
+            return rocfft_status_success;
+        }
+
+        const uint64_t n0   = p.len[0];
+        const uint64_t h0   = n0 / 2 + 1;
+        const bool     even = n0 % 2 == 0;
+        size_t         hlen[3];
+        for(size_t d = 0; d < 3; ++d)
+            hlen[d] = d < p.rank ? p.len[d] : 1;
+        hlen[0] = h0;
+
+        if(p.type == rocfft_transform_type_real_forward)
+        {
+            View hv = complex_view(out_buf, p.out_type, p.ostride, p.odist, p.ooffset, p.rank);
+            bool last0 = p.rank == 1;
+            if(even && n0 >= 2)
+            {
+                uint64_t half = n0 / 2;
+                View     rv   = realpair_view(BUF_IN, p.istride, p.idist, p.ioffset, p.rank);
+                auto     oth  = other_axes(rv, hv, p.len, p.rank, p.batch, 0);
+                if(single_kernel_length(half, b.esize))
+                {
+                    DimOps ops;
+                    ops.store_op = FFTK_STORE_R2C_POST;
+                    ops.half_tw  = half_twiddles(half, b.precision, b.dry);
+                    if(last0)
+                    {
+                        ops.scale     = p.scale;
+                        ops.has_scale = p.has_scale;
+                    }
+                    emit_dim(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, -1, ops);
+                }
+                else
+                {
+                    // half-length complex FFT into the output rows, then the
+                    // post-processing pass in place on those rows
+                    emit_dim(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, -1, DimOps());
+                    std::vector<Other> rows;
+                    for(const Other& o : oth)
+                        rows.push_back({o.cnt, o.os, o.os});
+                    emit_real_step(b, PASS_REAL_POST, half, rows, hv.stride[0], hv.io, hv.stride[0],
+                                   hv.io, p.scale, last0 && p.has_scale);
+                }
+            }
+            else
+            {
+                View   rv  = real_view(BUF_IN, p.istride, p.idist, p.ioffset, p.rank);
+                auto   oth = other_axes(rv, hv, p.len, p.rank, p.batch, 0);
+                DimOps ops;
+                ops.load_op         = FFTK_LOAD_REAL;
+                ops.src_real_scalar = true;
+                ops.n_out           = (uint32_t)h0;
+                if(last0)
+                {
+                    ops.scale     = p.scale;
+                    ops.has_scale = p.has_scale;
+                }
+                emit_dim(b, n0, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, -1, ops);
+            }
+            for(size_t d = 1; d < p.rank; ++d)
+            {
+                DimOps ops = d + 1 == p.rank ? scale_ops : DimOps();
+                emit_dim(b, p.len[d], hv.stride[d], hv.stride[d],
+                         other_axes(hv, hv, hlen, p.rank, p.batch, d), hv.io, hv.io, -1, ops);
+            }
+            return rocfft_status_success;
+        }
+
+        // real inverse: higher dimensions first, in place on the Hermitian input
+        // (an out-of-place real inverse may overwrite its input: reference
+        // rocfft.h:107-112, library/src/assignment_policy.cpp:601-606), then dimension 0
+        View hv = complex_view(BUF_IN, p.in_type, p.istride, p.idist, p.ioffset, p.rank);
+        for(size_t d = p.rank; d-- > 1;)
+            emit_dim(b, p.len[d], hv.stride[d], hv.stride[d],
+                     other_axes(hv, hv, hlen, p.rank, p.batch, d), hv.io, hv.io, +1, DimOps());
+        if(even && n0 >= 2)
+        {
+            uint64_t half = n0 / 2;
+            View     rv   = realpair_view(out_buf, p.ostride, p.odist, p.ooffset, p.rank);
+            auto     oth  = other_axes(hv, rv, p.len, p.rank, p.batch, 0);
+            if(single_kernel_length(half, b.esize))
+            {
+                DimOps ops;
+                ops.load_op   = FFTK_LOAD_C2R_PRE;
+                ops.half_tw   = half_twiddles(half, b.precision, b.dry);
+                ops.scale     = p.scale;
+                ops.has_scale = p.has_scale;
+                emit_dim(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io, +1, ops);
+            }
+            else
+            {
+                // pre-process into the output rows (viewed as half-length complex),
+                // then the half-length inverse FFT in place there
+                if(plan.inplace)
+                {
+                    bool same = !hv.io.planar && hv.stride[0] == rv.stride[0] && rv.io.im_delta == 1;
+                    for(int d = 1; d < 4; ++d)
+                        same = same && hv.stride[d] == rv.stride[d];
+                    if(!same)
+                        fail("in-place real inverse needs the standard padded layout");
+                }
+                std::vector<Other> rows;
+                for(const Other& o : oth)
+                    rows.push_back({o.cnt, o.os, o.is});
+                emit_real_step(b, PASS_REAL_PRE, half, rows, rv.stride[0], rv.io, hv.stride[0], hv.io,
+                               1.0, false);
+                std::vector<Other> oo;
+                for(const Other& o : oth)
+                    oo.push_back({o.cnt, o.os, o.os});
+                emit_dim(b, half, rv.stride[0], rv.stride[0], oo, rv.io, rv.io, +1, scale_ops);
+            }
+        }
+        else
+        {
+            View   rv  = real_view(out_buf, p.ostride, p.odist, p.ooffset, p.rank);
+            auto   oth = other_axes(hv, rv, p.len, p.rank, p.batch, 0);
+            DimOps ops;
+            ops.load_op         = FFTK_LOAD_HERM_EXPAND;
+            ops.store_op        = FFTK_STORE_REAL;
+            ops.dst_real_scalar = true;
+            ops.n_in            = (uint32_t)n0;
+            ops.scale           = p.scale;
+            ops.has_scale       = p.has_scale;
+            emit_dim(b, n0, hv.stride[0], rv.stride[0], oth, hv.io, rv.io, +1, ops);
+        }
+        return rocfft_status_success;
+    }
+    catch(const PlanError& e)
+    {
+        err = e.what();
+        return e.status;
+    }
+    catch(const std::exception& e)
+    {
+        err = e.what();
+        return rocfft_status_failure;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// executor (reference: TransformPowX, library/src/powX.cpp:525-957)
+
+static bool aligned(const void* p, size_t a)
+{
+    return ((uintptr_t)p % a) == 0;
+}
+
+rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
+                            void* stream)
+{
+    const size_t scalar = plan.precision ? 8 : 4;
+    char*        tmp    = static_cast<char*>(work);
+    char*        blu    = tmp ? tmp + plan.tmp_elems * plan.elem_bytes : nullptr;
+    auto resolve = [&](const IoRef& io, char*& p0, char*& p1) -> bool {
+        char* base0 = nullptr;
+        char* base1 = nullptr;
+        switch(io.buf)
+        {
+        case BUF_IN:
+            base0 = static_cast<char*>(in[0]);
+            base1 = static_cast<char*>(in[1]);
+            break;
+        case BUF_OUT:
+            base0 = static_cast<char*>(out[0]);
+            base1 = static_cast<char*>(out[1]);
+            break;
+        case BUF_TMP:
+            base0 = tmp;
+            break;
+        default:
+            base0 = blu;
+            break;
+        }
+        if(!base0)
+            return false;
+        p0 = base0 + io.off0 * (int64_t)scalar;
+        if(io.planar)
+        {
+            if(!base1)
+                return false;
+            p1 = base1 + io.off1 * (int64_t)scalar;
+        }
+        else
+            p1 = p0 + io.im_delta * (int64_t)scalar;
+        return true;
+    };
+    for(const PassRec& rec : plan.passes)
+    {
+        char *s0, *s1, *d0, *d1;
+        if(!resolve(rec.src, s0, s1) || !resolve(rec.dst, d0, d1))
+            return rocfft_status_failure;
+        int rc;
+        if(rec.kind == PASS_TILE)
+        {
+            fftk_params k = rec.kp;
+            k.in0         = s0;
+            k.in1         = s1;
+            k.out0        = d0;
+            k.out1        = d1;
+            bool vec = rec.vec_ok && aligned(s0, plan.elem_bytes) && aligned(d0, plan.elem_bytes);
+            rc = fftrt_launch_tile(&k, plan.precision, vec ? 1 : 0, rec.grid, rec.lds, stream);
+        }
+        else
+        {
+            fftk_real_params r = rec.rp;
+            if(rec.kind == PASS_REAL_POST)
+            {
+                r.z0  = s0;
+                r.z1  = s1;
+                r.ho0 = d0;
+                r.ho1 = d1;
+                rc    = fftrt_launch_real_post(&r, plan.precision, stream);
+            }
+            else
+            {
+                r.h0  = s0;
+                r.h1  = s1;
+                r.zo0 = d0;
+                r.zo1 = d1;
+                rc    = fftrt_launch_real_pre(&r, plan.precision, stream);
+            }
+        }
+        if(rc != 0)
+            return rocfft_status_failure;
+    }
+    return rocfft_status_success;
+}
+
+static const char* buf_name(int b)
+{
+    switch(b)
+    {
+    case BUF_IN:
+        return "in";
+    case BUF_OUT:
+        return "out";
+    case BUF_TMP:
+        return "tmp";
+    default:
+        return "blu";
+    }
+}
+
+std::string ExecPlan::describe() const
+{
+    std::ostringstream o;
+    o << "plan: " << passes.size() << " passes, precision " << (precision ? "double" : "single")
+      << ", work buffer " << work_bytes() << " bytes\n";
+    int i = 0;
+    for(const PassRec& r : passes)
+    {
+        o << "  pass " << i++ << ": " << r.note << " [" << buf_name(r.src.buf) << " -> "
+          << buf_name(r.dst.buf) << "]";
+        if(r.kind == PASS_TILE)
+        {
+            const fftk_params& k = r.kp;
+            o << " radix";
+            for(uint32_t p = 0; p < k.nf; ++p)
+                o << (p ? "x" : " ") << k.radix[p];
+            o << " tile " << k.W << "x" << k.n << " threads " << k.nthreads << " grid " << r.grid
+              << " lds " << r.lds << " in_fast_" << (k.in_fast_tile ? "tile" : "fft") << " out_fast_"
+              << (k.out_fast_tile ? "tile" : "fft") << " flags 0x" << std::hex << k.flags << std::dec
+              << " load " << k.load_op << " store " << k.store_op << (r.vec_ok ? " vec" : " scalar");
+        }
+        else
+            o << " half " << r.rp.half << " rows " << r.rp.rows0 << "x" << r.rp.rows1 << "x"
+              << r.rp.rows2;
+        o << "\n";
+    }
+    return o.str();
+}
+
+} // namespace fftamd

@@ -1,0 +1,114 @@
+// plan.h -- host-side plan model: a transform becomes a short list of passes,
+// each one launch of a precompiled kernel.  Plain C++, no HIP types; the GPU is
+// reached only through gpu_rt.h.
+//
+// Reference counterparts: the tree of TreeNode/LeafNode objects and ExecPlan
+// (library/src/include/tree_node.h:254-673, :1220-1323) built by
+// NodeFactory (library/src/node_factory.cpp:474-834) and executed by
+// TransformPowX (library/src/powX.cpp:525-957).  This planner emits the leaf
+// sequence directly instead of building and then fusing a tree.
+#ifndef ROCFFT_AMD_PLAN_H
+#define ROCFFT_AMD_PLAN_H
+
+#include "kparams.h"
+#include "rocfft/rocfft.h"
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace fftamd
+{
+
+enum BufId
+{
+    BUF_IN  = 0, // user input
+    BUF_OUT = 1, // user output
+    BUF_TMP = 2, // work buffer, general scratch region
+    BUF_BLU = 3  // work buffer, Bluestein region
+};
+
+// a device-resident table, shared between plans through the table cache
+struct DeviceTable
+{
+    void*  dptr  = nullptr;
+    size_t bytes = 0;
+    ~DeviceTable();
+};
+typedef std::shared_ptr<DeviceTable> TablePtr;
+
+// the transform as the API describes it, after defaults have been filled in
+struct Problem
+{
+    rocfft_transform_type   type;
+    rocfft_precision        precision;
+    rocfft_result_placement placement;
+    size_t                  rank;
+    size_t                  len[3]; // transform lengths (real lengths for real transforms)
+    size_t                  batch;
+    rocfft_array_type       in_type, out_type;
+    size_t                  istride[3], ostride[3], idist, odist;
+    size_t                  ioffset[2], ooffset[2];
+    double                  scale;
+    bool                    has_scale;
+};
+
+enum PassKind
+{
+    PASS_TILE      = 0,
+    PASS_REAL_POST = 1,
+    PASS_REAL_PRE  = 2
+};
+
+// where a pass finds one side of its data: buffer, planar or not, scalar offsets
+struct IoRef
+{
+    int     buf      = BUF_IN;
+    bool    planar   = false;
+    int64_t im_delta = 1; // scalars from a real part to its imaginary part (non planar)
+    int64_t off0     = 0; // scalar offset of the first element (real-part array)
+    int64_t off1     = 0; // scalar offset in the imaginary-part array (planar)
+};
+
+struct PassRec
+{
+    PassKind              kind = PASS_TILE;
+    fftk_params           kp;
+    fftk_real_params      rp;
+    IoRef                 src, dst;
+    bool                  vec_ok = false;
+    uint32_t              grid   = 0;
+    size_t                lds    = 0;
+    std::string           note;
+    std::vector<TablePtr> tables; // keeps the device tables alive
+};
+
+struct ExecPlan
+{
+    std::vector<PassRec> passes;
+    int                  precision  = 0; // 0 float, 1 double
+    size_t               tmp_elems  = 0; // complex elements of general scratch
+    size_t               blu_elems  = 0; // complex elements of Bluestein scratch
+    size_t               elem_bytes = 8; // bytes per complex element
+    bool                 inplace    = false;
+    size_t               work_bytes() const
+    {
+        return (tmp_elems + blu_elems) * elem_bytes;
+    }
+    std::string describe() const;
+};
+
+// Builds the pass list.  With dry_run no device memory is touched (tables get
+// null device pointers), so the planner can be exercised without a GPU.
+rocfft_status build_exec_plan(const Problem& prob, ExecPlan& plan, bool dry_run, std::string& err);
+
+// Enqueues every pass on `stream`.  in/out hold one pointer (interleaved, real)
+// or two (planar).  `work` must hold plan.work_bytes() bytes when that is non-zero.
+rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
+                            void* stream);
+
+// drops cached tables that no plan uses any more
+void table_cache_clear();
+
+} // namespace fftamd
+
+#endif
