@@ -1,0 +1,356 @@
+"""GPU parity tests: the HIP library, called through its C ABI, against the CPU
+checker on the same seeded inputs, against the committed golden fixtures, and --
+at the full benchmark sizes -- through size-independent properties (unnormalised
+round trip, Parseval, spot bins evaluated from the DFT definition) plus a
+cross-check against torch.fft, which on ROCm is the reference rocFFT behind
+hipFFT.
+
+Tolerances are the north-star bar: relative L2 and Linf <= 1e-5 in single and
+<= 1e-13 in double precision (helpers.tolerance).
+"""
+import os
+import threading
+
+import numpy as np
+import pytest
+
+import helpers as H
+import inputs
+import rocfft_amd.binding as B
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def gpu(gpu_lib):
+    return gpu_lib, H.TorchBackend()
+
+
+def tnorm(torch, a, b):
+    """(rel L2, rel Linf) of a against b, both device tensors, over all scalars"""
+    a = torch.view_as_real(a) if a.is_complex() else a
+    b = torch.view_as_real(b) if b.is_complex() else b
+    d = (a.double() - b.double())
+    l2 = (torch.linalg.vector_norm(d) / torch.linalg.vector_norm(b.double())).item()
+    li = (d.abs().max() / b.double().abs().max()).item()
+    return l2, li
+
+
+# ------------------------------------------------------------------ against the checker
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 16, 30, 64, 100, 128, 256, 512, 1000, 1024, 2048, 4096,
+                               8192, 11, 13, 17, 97, 121, 1001, 2310])
+def test_c2c_1d(gpu, n):
+    lib, be = gpu
+    for prec in (B.SINGLE, B.DOUBLE):
+        H.check(lib, be, B.COMPLEX_FORWARD, [n], 5, prec)
+        H.check(lib, be, B.COMPLEX_INVERSE, [n], 3, prec, inplace=True)
+
+
+@pytest.mark.parametrize("n", [2, 4, 6, 8, 30, 64, 256, 1000, 4096, 8192, 3, 9, 15, 17, 34, 97, 194])
+def test_real_1d(gpu, n):
+    lib, be = gpu
+    for prec in (B.SINGLE, B.DOUBLE):
+        for kind in (B.REAL_FORWARD, B.REAL_INVERSE):
+            H.check(lib, be, kind, [n], 5, prec)
+            H.check(lib, be, kind, [n], 2, prec, inplace=True)
+
+
+@pytest.mark.parametrize("n", [16384, 32768, 65536, 2 ** 18, 2 ** 20, 6000, 30030, 10007, 4099, 8198, 65537])
+def test_long_1d(gpu, n):
+    lib, be = gpu
+    H.check(lib, be, B.COMPLEX_FORWARD, [n], 3, B.SINGLE)
+    H.check(lib, be, B.COMPLEX_INVERSE, [n], 2, B.DOUBLE, inplace=True)
+    if n % 2 == 0:
+        H.check(lib, be, B.REAL_FORWARD, [n], 3, B.DOUBLE)
+        H.check(lib, be, B.REAL_INVERSE, [n], 3, B.SINGLE)
+        H.check(lib, be, B.REAL_FORWARD, [n], 2, B.SINGLE, inplace=True)
+        H.check(lib, be, B.REAL_INVERSE, [n], 2, B.DOUBLE, inplace=True)
+
+
+@pytest.mark.parametrize("lengths", [[8, 8], [64, 64], [100, 30], [17, 19], [1024, 1024], [4096, 64], [64, 4096],
+                                     [8, 8, 8], [16, 8, 4], [30, 20, 10], [128, 32, 8], [5, 7, 9], [64, 64, 64],
+                                     [128, 128, 128], [512, 16, 16], [16, 512, 4], [8, 4, 512], [1, 8], [8, 1, 4]])
+def test_multi_dim(gpu, lengths):
+    lib, be = gpu
+    for kind in range(4):
+        H.check(lib, be, kind, lengths, 2, B.DOUBLE)
+        H.check(lib, be, kind, lengths, 1, B.SINGLE, inplace=True)
+
+
+def test_layouts(gpu):
+    lib, be = gpu
+    K = B
+    H.check(lib, be, K.COMPLEX_FORWARD, [64], 3, K.DOUBLE, in_strides=[3], in_dist=200, out_strides=[2],
+            out_dist=130, in_offsets=[5, 0], out_offsets=[7, 0])
+    H.check(lib, be, K.COMPLEX_FORWARD, [128], 8, K.SINGLE, in_strides=[8], in_dist=1, out_strides=[8],
+            out_dist=1)
+    H.check(lib, be, K.COMPLEX_INVERSE, [30, 4], 2, K.DOUBLE, in_type=K.COMPLEX_PLANAR,
+            out_type=K.COMPLEX_PLANAR, in_offsets=[3, 9], out_offsets=[2, 1])
+    H.check(lib, be, K.COMPLEX_FORWARD, [16384], 2, K.SINGLE, in_type=K.COMPLEX_INTERLEAVED,
+            out_type=K.COMPLEX_PLANAR)
+    H.check(lib, be, K.REAL_FORWARD, [32, 6], 2, K.DOUBLE, out_type=K.HERMITIAN_PLANAR)
+    H.check(lib, be, K.REAL_INVERSE, [32, 6], 2, K.DOUBLE, in_type=K.HERMITIAN_PLANAR)
+    H.check(lib, be, K.REAL_FORWARD, [20, 6], 2, K.SINGLE, in_strides=[1, 23], in_dist=150,
+            out_strides=[1, 13], out_dist=90)
+    H.check(lib, be, K.REAL_INVERSE, [21, 6], 2, K.SINGLE, in_strides=[2, 30], in_dist=200,
+            out_strides=[1, 25], out_dist=160)
+    H.check(lib, be, K.COMPLEX_FORWARD, [16, 8], 2, K.DOUBLE, out_strides=[8, 1], out_dist=128)
+    for kind, lengths in [(0, [64]), (1, [16384]), (2, [64]), (2, [16384]), (3, [64]), (3, [16384]), (0, [97]),
+                          (0, [4099]), (0, [8, 8, 8]), (2, [8, 8]), (3, [7, 8])]:
+        H.check(lib, be, kind, lengths, 2, K.DOUBLE, scale=1.0 / 64)
+
+
+def test_no_stray_writes(gpu):
+    lib, be = gpu
+    for kind, lengths, kw in [(0, [64], dict(out_strides=[3], out_dist=250)),
+                              (0, [16384], dict(out_strides=[2], out_dist=40000)),
+                              (2, [30, 4], dict(out_strides=[2, 40], out_dist=200)),
+                              (3, [32, 4], dict(out_strides=[1, 37], out_dist=170)),
+                              (0, [97], dict(out_strides=[2], out_dist=300))]:
+        y, x, touched = H.run_transform(lib, be, kind, lengths, 2, B.SINGLE, return_buffers=True, **kw)
+        for raw, mask in touched:
+            assert np.all(raw[~mask[:raw.size]] == H.GUARD), (kind, lengths)
+        assert orc.rel_norms(y, H.reference(kind, lengths, 2, x, B.SINGLE))[0] < 1e-5
+
+
+def test_c2r_ignores_imaginary_dc_and_nyquist(gpu):
+    lib, be = gpu
+    for n in (8, 8192, 65536, 9):
+        h = H.make_input(B.REAL_INVERSE, [n], 1)
+        h2 = h.copy()
+        h2[0, 0] += 2.5j
+        if n % 2 == 0:
+            h2[0, -1] -= 1.5j
+        y1, _ = H.run_transform(lib, be, B.REAL_INVERSE, [n], 1, B.DOUBLE, x=h)
+        y2, _ = H.run_transform(lib, be, B.REAL_INVERSE, [n], 1, B.DOUBLE, x=h2)
+        assert np.array_equal(y1, y2), n
+
+
+def test_work_buffer_contract(gpu):
+    lib, be = gpu
+    torch = be.torch
+    n = 8191
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], 1, lib=lib)
+    need = plan.work_buffer_size
+    assert need > 0
+    x = torch.zeros(n, dtype=torch.complex64, device=be.dev)
+    x[1] = 1
+    y = torch.zeros_like(x)
+    plan.execute([x.data_ptr()], [y.data_ptr()])  # scratch allocated by execute
+    torch.cuda.synchronize()
+    want = np.exp(-2j * np.pi * np.arange(n) / n)
+    assert np.allclose(y.cpu().numpy(), want, atol=1e-4)
+    info = B.ExecutionInfo(lib)
+    small = torch.zeros(need // 2, dtype=torch.uint8, device=be.dev)
+    info.set_work_buffer(small.data_ptr(), need // 2)
+    assert plan.execute_status([x.data_ptr()], [y.data_ptr()], info) == B.STATUS_INVALID_WORK_BUFFER
+
+
+def test_streams_threads_and_graph_capture(gpu):
+    lib, be = gpu
+    torch = be.torch
+    n, batch = 4096, 64
+    x = inputs.torch_uniform01(torch, be.dev, 5, 0, 2 * n * batch).to(torch.float32) - 0.5
+    x = torch.view_as_complex(x.reshape(batch, n, 2).contiguous())
+    ref = torch.fft.fft(x, dim=1)
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], batch, lib=lib)
+    # several user streams (reference clients/tests/multithread_test.cpp:310-348)
+    outs, streams = [], [torch.cuda.Stream() for _ in range(3)]
+    torch.cuda.synchronize()
+    for s in streams:
+        y = torch.empty_like(x)
+        info = B.ExecutionInfo(lib).set_stream(s.cuda_stream)
+        plan.execute([x.data_ptr()], [y.data_ptr()], info)
+        outs.append(y)
+    torch.cuda.synchronize()
+    for y in outs:
+        assert tnorm(torch, y, ref)[0] < 1e-5
+    # plan creation and execution from several host threads (multithread_test.cpp:255-278)
+    errs = []
+
+    def worker(k):
+        try:
+            p = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n >> k], batch << k, lib=lib)
+            s = torch.cuda.Stream()
+            y = torch.empty_like(x)
+            p.execute([x.data_ptr()], [y.data_ptr()], B.ExecutionInfo(lib).set_stream(s.cuda_stream))
+            s.synchronize()
+            want = torch.fft.fft(x.reshape(batch << k, n >> k), dim=1)
+            if tnorm(torch, y.reshape(batch << k, n >> k), want)[0] > 1e-5:
+                errs.append(k)
+        except Exception as e:  # noqa: BLE001
+            errs.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(4)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    assert not errs, errs
+    # rocfft_execute can be captured into a graph and replayed (clients/tests/hipGraph_test.cpp:272)
+    y = torch.zeros_like(x)
+    xin = x.clone()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            info = B.ExecutionInfo(lib).set_stream(torch.cuda.current_stream().cuda_stream)
+            plan.execute([xin.data_ptr()], [y.data_ptr()], info)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        xin.copy_(x * (rep + 1))
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert tnorm(torch, y, ref * (rep + 1))[0] < 1e-5, rep
+
+
+# ------------------------------------------------------------------ the five configurations, full size
+def golden_check(cfg_id, y_rows):
+    g = np.load(os.path.join(GOLDEN, "cfg%d.npz" % cfg_id))
+    rows = int(g["rows"])
+    y = y_rows[:rows]
+    scale = g["l2"][:rows, None] / np.sqrt(y.shape[1])
+    tol = H.tolerance(B.SINGLE if inputs.CONFIGS[cfg_id]["precision"] == "single" else B.DOUBLE)
+    err = np.max(np.abs(y[:, g["bins"]] - g["values"][:rows]) / scale)
+    assert err < 10 * tol, err  # a single bin against the rms bin magnitude
+    assert np.max(np.abs(np.sqrt((np.abs(y) ** 2).sum(axis=1)) / g["l2"][:rows] - 1)) < tol
+
+
+def run_plan(lib, torch, plan, src, dst):
+    info = B.ExecutionInfo(lib)
+    wb = plan.work_buffer_size
+    work = None
+    if wb:
+        work = torch.empty(wb, dtype=torch.uint8, device=src.device)
+        info.set_work_buffer(work.data_ptr(), wb)
+    plan.execute([src.data_ptr()], None if dst is None else [dst.data_ptr()], info)
+    torch.cuda.synchronize()
+
+
+def test_config1_c2c_4096_inplace(gpu):
+    lib, be = gpu
+    torch = be.torch
+    x = inputs.torch_config_input(torch, be.dev, 1)
+    buf = x.clone()
+    plan = B.Plan(B.INPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4096], 1024, lib=lib)
+    run_plan(lib, torch, plan, buf, None)
+    y = buf.cpu().numpy().astype(np.complex128)
+    ref = orc.transform(orc.COMPLEX_FORWARD, [4096], 1024, x.cpu().numpy().astype(np.complex128))
+    l2, li = orc.rel_norms(y.reshape(-1), ref)
+    assert l2 <= 1e-5 and li <= 1e-5, (l2, li)
+    golden_check(1, y)
+    assert tnorm(torch, buf, torch.fft.fft(x, dim=1))[0] <= 1e-5  # reference rocFFT via hipFFT
+
+
+def test_config2_r2c_c2r_65536(gpu):
+    lib, be = gpu
+    torch = be.torch
+    n, batch = 65536, 4096
+    x = inputs.torch_config_input(torch, be.dev, 2)
+    keep = x.clone()
+    h = torch.empty((batch, n // 2 + 1), dtype=torch.complex64, device=be.dev)
+    fwd = B.Plan(B.NOTINPLACE, B.REAL_FORWARD, B.SINGLE, [n], batch, lib=lib)
+    run_plan(lib, torch, fwd, x, h)
+    assert torch.equal(x, keep)  # out-of-place forward keeps its input
+    head = h[:8].cpu().numpy().astype(np.complex128)
+    ref = orc.transform(orc.REAL_FORWARD, [n], 8, x[:8].cpu().numpy().astype(np.float64)).reshape(8, -1)
+    l2, li = orc.rel_norms(head, ref)
+    assert l2 <= 1e-5 and li <= 1e-5, (l2, li)
+    golden_check(2, head)
+    assert tnorm(torch, h, torch.fft.rfft(x, dim=1))[0] <= 1e-5
+    assert h[:, 0].imag.abs().max().item() == 0 and h[:, -1].imag.abs().max().item() == 0
+    # Parseval over the whole batch: sum |x|^2 * n = |X0|^2 + |Xnyq|^2 + 2 sum_{0<k<n/2} |Xk|^2
+    e_in = (x.double() ** 2).sum().item() * n
+    hh = h.abs().double() ** 2
+    e_out = (2 * hh.sum() - hh[:, 0].sum() - hh[:, -1].sum()).item()
+    assert abs(e_out / e_in - 1) < 1e-5
+    # unnormalised round trip (reference shared/accuracy_test.h:685-861)
+    back = torch.empty_like(x)
+    inv = B.Plan(B.NOTINPLACE, B.REAL_INVERSE, B.SINGLE, [n], batch, lib=lib)
+    run_plan(lib, torch, inv, h, back)
+    l2, li = tnorm(torch, back / n, x)
+    assert l2 <= 1e-5 and li <= 1e-5, (l2, li)
+
+
+def test_config3_c2c_4096x4096(gpu):
+    lib, be = gpu
+    torch = be.torch
+    x = inputs.torch_config_input(torch, be.dev, 3)
+    keep = x.clone()
+    y = torch.empty_like(x)
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4096, 4096], 8, lib=lib)
+    run_plan(lib, torch, plan, x, y)
+    assert torch.equal(x, keep)
+    golden_check(3, y[:1].cpu().numpy().astype(np.complex128))
+    ref = torch.fft.fft2(x.reshape(8, 4096, 4096)).reshape(8, -1)
+    l2, li = tnorm(torch, y, ref)
+    assert l2 <= 1e-5 and li <= 1e-5, (l2, li)
+    del ref
+    # spot bins of the last batch entry from the 2D DFT definition (separable: rows then one column sum)
+    xb = x[7].reshape(4096, 4096).cpu().numpy().astype(np.complex128)
+    for (k1, k0) in [(0, 0), (1, 4095), (2049, 77)]:
+        col = (xb * np.exp(-2j * np.pi * k0 * np.arange(4096) / 4096)[None, :]).sum(axis=1)
+        want = orc.dft_bin(col, k1)
+        got = complex(y[7, k1 * 4096 + k0].item())
+        assert abs(got - want) / 4096 < 1e-4
+    # round trip
+    back = torch.empty_like(x)
+    inv = B.Plan(B.NOTINPLACE, B.COMPLEX_INVERSE, B.SINGLE, [4096, 4096], 8, lib=lib)
+    run_plan(lib, torch, inv, y, back)
+    l2, li = tnorm(torch, back / (4096.0 * 4096.0), x)
+    assert l2 <= 1e-5 and li <= 1e-5, (l2, li)
+
+
+def test_config4_r2c_c2r_512cubed_double(gpu):
+    lib, be = gpu
+    torch = be.torch
+    n = 512
+    x = inputs.torch_config_input(torch, be.dev, 4)
+    keep = x.clone()
+    h = torch.empty((1, n * n * (n // 2 + 1)), dtype=torch.complex128, device=be.dev)
+    fwd = B.Plan(B.NOTINPLACE, B.REAL_FORWARD, B.DOUBLE, [n, n, n], 1, lib=lib)
+    run_plan(lib, torch, fwd, x, h)
+    assert torch.equal(x, keep)
+    golden_check(4, h.cpu().numpy())
+    ref = torch.fft.rfftn(x.reshape(n, n, n)).reshape(1, -1)
+    l2, li = tnorm(torch, h, ref)
+    assert l2 <= 1e-13 and li <= 1e-13, (l2, li)
+    del ref
+    back = torch.empty_like(x)
+    inv = B.Plan(B.NOTINPLACE, B.REAL_INVERSE, B.DOUBLE, [n, n, n], 1, lib=lib)
+    run_plan(lib, torch, inv, h.clone(), back)  # the inverse may overwrite its input
+    l2, li = tnorm(torch, back / float(n ** 3), x)
+    assert l2 <= 1e-13 and li <= 1e-13, (l2, li)
+
+
+def test_config5_bluestein_prime_1000003_double(gpu):
+    lib, be = gpu
+    torch = be.torch
+    n, batch = 1000003, 16
+    x = inputs.torch_config_input(torch, be.dev, 5)
+    keep = x.clone()
+    y = torch.empty_like(x)
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.DOUBLE, [n], batch, lib=lib)
+    run_plan(lib, torch, plan, x, y)
+    assert torch.equal(x, keep)
+    yh = y.cpu().numpy()
+    golden_check(5, yh)
+    # full comparison of two rows with the long double checker, spot bins on the others
+    xh = x.cpu().numpy()
+    ref = orc.fft1d(xh[:2], ld=True)
+    l2, li = orc.rel_norms(yh[:2], ref)
+    assert l2 <= 1e-13 and li <= 1e-13, (l2, li)
+    scale = np.abs(yh).max()
+    for b in (2, 9, 15):
+        for k in (0, 1, 500001, n - 1):
+            assert abs(yh[b, k] - orc.dft_bin(xh[b], k)) / scale < 1e-13
+    l2, li = tnorm(torch, y, torch.fft.fft(x, dim=1))
+    assert l2 <= 1e-13, (l2, li)  # reference rocFFT; its own error is in this figure too
+    back = torch.empty_like(x)
+    inv = B.Plan(B.NOTINPLACE, B.COMPLEX_INVERSE, B.DOUBLE, [n], batch, lib=lib)
+    run_plan(lib, torch, inv, y, back)
+    l2, li = tnorm(torch, back / float(n), x)
+    assert l2 <= 1e-13 and li <= 1e-13, (l2, li)
