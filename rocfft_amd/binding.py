@@ -100,6 +100,13 @@ class Library:
                 "%s is missing: build it with __graft_entry__.build() (hipcc, gfx950); "
                 "there is no fallback implementation" % path)
         self.path = path
+        # PyTorch wheels carry their own copy of the HIP runtime under the same soname.
+        # When a process uses both, torch must be loaded first so that this library
+        # binds to the runtime torch initialises (one runtime per process).
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         self.c = ctypes.CDLL(path)
         for name, args in _PROTOTYPES.items():
             fn = getattr(self.c, name)
