@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the FFT hot path on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic input that
+is already resident in HBM: for the default workload (the second benchmark
+configuration) a step is the real forward transform of 4096 signals of 65536
+float32 samples followed by the real inverse transform of the result, both out
+of place, through rocfft_execute of this library's C ABI.
+
+Prints ONE JSON line.  `value` is GFLOP/s in the 5*N*log2(N) convention summed
+over the transforms of a step.  `roofline` prices the slowest kernel of the step
+against the HBM peak using per-kernel durations taken with HIP events inside this
+script; `cpu_baseline` times the CPU checker (a port of the algorithm, OpenMP
+across the batch) on a bounded sample of the same workload.  `all_configs` adds
+one short measurement for each of the five benchmark configurations, next to
+torch.fft on the same device (on ROCm that is the reference rocFFT behind
+hipFFT), as reported baselines.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+
+def workloads():
+    """name, transform list [(kind, lengths, batch, precision, inplace)], flops and bytes per step"""
+    import rocfft_amd as rf
+
+    def flops(lengths, batch):
+        n = 1
+        for v in lengths:
+            n *= v
+        return 5.0 * n * math.log2(n) * batch
+
+    w = {}
+    n, b = 4096, 1024
+    w[1] = dict(name="c2c_1d_4096_x1024_f32_inplace", dtype="f32",
+                transforms=[(rf.COMPLEX_FORWARD, [n], b, rf.SINGLE, True)], flops=flops([n], b),
+                bytes=2.0 * n * b * 8)
+    n, b = 65536, 4096
+    per_dir = n * b * 4 + (n // 2 + 1) * b * 8
+    w[2] = dict(name="r2c_c2r_1d_65536_x4096_f32_roundtrip", dtype="f32",
+                transforms=[(rf.REAL_FORWARD, [n], b, rf.SINGLE, False), (rf.REAL_INVERSE, [n], b, rf.SINGLE, False)],
+                flops=2 * flops([n], b), bytes=2.0 * per_dir)
+    n, b = 4096, 8
+    w[3] = dict(name="c2c_2d_4096x4096_x8_f32", dtype="f32",
+                transforms=[(rf.COMPLEX_FORWARD, [n, n], b, rf.SINGLE, False)], flops=flops([n, n], b),
+                bytes=2.0 * n * n * b * 8)
+    n = 512
+    per_dir = n ** 3 * 8 + n * n * (n // 2 + 1) * 16
+    w[4] = dict(name="r2c_c2r_3d_512cubed_f64_roundtrip", dtype="f64",
+                transforms=[(rf.REAL_FORWARD, [n, n, n], 1, rf.DOUBLE, False),
+                            (rf.REAL_INVERSE, [n, n, n], 1, rf.DOUBLE, False)],
+                flops=2 * flops([n, n, n], 1), bytes=2.0 * per_dir)
+    n, b = 1000003, 16
+    w[5] = dict(name="c2c_1d_prime1000003_x16_f64_bluestein", dtype="f64",
+                transforms=[(rf.COMPLEX_FORWARD, [n], b, rf.DOUBLE, False)], flops=flops([n], b),
+                bytes=2.0 * n * b * 16)
+    return w
+
+
+class Step:
+    """plans, device buffers and execution infos of one workload; run() enqueues one step"""
+
+    def __init__(self, cfg_id, wl, torch, stream_ptr):
+        import inputs
+        import rocfft_amd as rf
+
+        self.torch = torch
+        self.rf = rf
+        dev = torch.device("cuda:0")
+        self.x = inputs.torch_config_input(torch, dev, cfg_id).contiguous()
+        self.calls = []
+        self.keep = []
+        cur = self.x
+        for (kind, lengths, batch, prec, inplace) in wl["transforms"]:
+            plan = rf.Plan(rf.INPLACE if inplace else rf.NOTINPLACE, kind, prec, lengths, batch)
+            rt = torch.float32 if prec == rf.SINGLE else torch.float64
+            ct = torch.complex64 if prec == rf.SINGLE else torch.complex128
+            total = 1
+            for v in lengths:
+                total *= v
+            h = total // lengths[0] * (lengths[0] // 2 + 1)
+            if inplace:
+                out = None
+            elif kind == rf.REAL_FORWARD:
+                out = torch.empty((batch, h), dtype=ct, device=dev)
+            elif kind == rf.REAL_INVERSE:
+                out = torch.empty((batch, total), dtype=rt, device=dev)
+            else:
+                out = torch.empty((batch, total), dtype=ct, device=dev)
+            info = rf.ExecutionInfo()
+            info.set_stream(stream_ptr)
+            wb = plan.work_buffer_size
+            if wb:
+                work = torch.empty(wb, dtype=torch.uint8, device=dev)
+                info.set_work_buffer(work.data_ptr(), wb)
+                self.keep.append(work)
+            self.calls.append((plan, cur, out, info))
+            cur = cur if inplace else out
+        self.result = cur
+
+    def run(self):
+        for plan, src, dst, info in self.calls:
+            plan.execute([src.data_ptr()], None if dst is None else [dst.data_ptr()], info)
+
+    def profile(self):
+        """[(pass name, bytes read+written, ms)] of one step, every kernel bracketed by events"""
+        rows = []
+        for plan, src, dst, info in self.calls:
+            ms = plan.execute_profile([src.data_ptr()], None if dst is None else [dst.data_ptr()], info)
+            for (name, nbytes), t in zip(plan.passes(), ms):
+                rows.append((name, nbytes, t))
+        return rows
+
+
+def time_steps(torch, step, warmup, steps):
+    for _ in range(warmup):
+        step.run()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        step.run()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    dev = start.elapsed_time(stop) / steps
+    # the driver checks against its own wall clock: report the larger of the two
+    return max(wall, dev), dev
+
+
+def kernel_profile(step, reps):
+    acc = None
+    for _ in range(reps):
+        rows = step.profile()
+        if acc is None:
+            acc = [[name, nbytes, 0.0] for name, nbytes, _ in rows]
+        for a, (_, _, t) in zip(acc, rows):
+            a[2] += t / reps
+    return acc
+
+
+def cpu_baseline(cfg_id, wl, budget_s=12.0):
+    """the CPU checker (double precision port, OpenMP over the batch) on a bounded sample"""
+    import numpy as np
+
+    import inputs
+    from oracle import oracle as orc
+
+    kinds = {0: orc.COMPLEX_FORWARD, 1: orc.COMPLEX_INVERSE, 2: orc.REAL_FORWARD, 3: orc.REAL_INVERSE}
+    full_batch = wl["transforms"][0][2]
+    lengths = wl["transforms"][0][1]
+
+    def run(nb):
+        x = inputs.config_input(cfg_id, 0, nb)
+        t0 = time.perf_counter()
+        cur = x
+        for (kind, ln, _, _, _) in wl["transforms"]:
+            cur = orc.transform(kinds[kind], ln, nb, cur, ld=False)
+        return time.perf_counter() - t0
+
+    threads = orc.num_threads()
+    nb = min(full_batch, max(1, threads))
+    t = run(nb)
+    target = int(min(full_batch, max(nb, nb * budget_s / max(t, 1e-6))))
+    target = max(threads, target // threads * threads) if full_batch >= threads else full_batch
+    target = min(target, full_batch)
+    if target > nb:
+        t = run(target)
+        nb = target
+    frac = nb / full_batch
+    return dict(value=wl["flops"] * frac / t / 1e9, unit="GFLOP/s", cores=threads, kind="port",
+                sample="%d of %d transforms of %s, %.1f s, oracle/fft_oracle.c double build, %d OpenMP threads"
+                % (nb, full_batch, "x".join(map(str, lengths)), t, threads))
+
+
+def reference_rocfft_ms(torch, cfg_id, step, reps=5):
+    """torch.fft on the same device buffers (reference rocFFT behind hipFFT); median ms per step"""
+    x = step.x
+
+    def run():
+        if cfg_id == 1:
+            return torch.fft.fft(x, dim=1)
+        if cfg_id == 2:
+            return torch.fft.irfft(torch.fft.rfft(x, dim=1), n=65536, dim=1, norm="forward")
+        if cfg_id == 3:
+            return torch.fft.fft2(x.reshape(8, 4096, 4096))
+        if cfg_id == 4:
+            return torch.fft.irfftn(torch.fft.rfftn(x.reshape(512, 512, 512)), s=(512, 512, 512), norm="forward")
+        return torch.fft.fft(x, dim=1)
+
+    try:
+        run()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            run()
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b))
+        ts.sort()
+        return ts[len(ts) // 2]
+    except Exception:  # noqa: BLE001  (a baseline, never fatal)
+        return None
+
+
+def measure_config(torch, cfg_id, wl, stream_ptr, warmup, steps, prof_reps):
+    step = Step(cfg_id, wl, torch, stream_ptr)
+    ms, dev_ms = time_steps(torch, step, warmup, steps)
+    prof = kernel_profile(step, prof_reps)
+    return step, ms, dev_ms, prof
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default 2)")
+    ap.add_argument("--no-extras", action="store_true", help="skip all_configs and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build drives one GPU; --gpus %d is not supported "
+              "(every transform of these workloads shards by batch without communication)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import rocfft_amd as rf
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU", file=sys.stderr)
+        sys.exit(1)
+    rf.library()  # raises if the HIP library is not built
+    stream_ptr = torch.cuda.current_stream().cuda_stream
+    wls = workloads()
+    wl = wls[args.config]
+
+    step, ms, dev_ms, prof = measure_config(torch, args.config, wl, stream_ptr, args.warmup, args.steps, 5)
+    dom = max(prof, key=lambda r: r[2])
+    achieved = dom[1] / (dom[2] * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(wl["name"], {}).get(dom[0])
+        except Exception:  # noqa: BLE001
+            traffic = None
+    out = {
+        "metric": "GFLOP/s (5N*log2N) per config, 1 GPU",
+        "value": wl["flops"] / (ms * 1e-3) / 1e9,
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": wl["dtype"],
+        "data": "synthetic",
+        "config": {"workload": wl["name"], "transforms_per_step": len(wl["transforms"]),
+                   "kernels_per_step": len(prof)},
+        "device_ms_per_step": dev_ms,
+        "algorithmic_GBps": wl["bytes"] / (ms * 1e-3) / 1e9,
+        "algorithmic_hbm_frac": wl["bytes"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": dom[0],
+                     "kernel_ms": dom[2], "kernel_bytes": dom[1]},
+        "kernels": [{"name": n, "bytes": b, "ms": t, "GBps": b / (t * 1e-3) / 1e9 if t > 0 else None}
+                    for n, b, t in prof],
+    }
+    if not args.no_extras:
+        ref_ms = reference_rocfft_ms(torch, args.config, step)
+        allc = {}
+        for cid in sorted(wls):
+            if cid == args.config:
+                s2, m2, p2 = step, ms, prof
+                r2 = ref_ms
+            else:
+                del step
+                torch.cuda.empty_cache()
+                s2, m2, _, p2 = measure_config(torch, cid, wls[cid], stream_ptr, 2, 10, 2)
+                r2 = reference_rocfft_ms(torch, cid, s2)
+                step = s2
+            w2 = wls[cid]
+            allc[w2["name"]] = {
+                "ms": m2, "GFLOPs": w2["flops"] / (m2 * 1e-3) / 1e9,
+                "GBps": w2["bytes"] / (m2 * 1e-3) / 1e9,
+                "hbm_frac": w2["bytes"] / (m2 * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "kernels": len(p2),
+                "reference_rocfft_ms": r2,
+                "reference_rocfft_GFLOPs": (w2["flops"] / (r2 * 1e-3) / 1e9) if r2 else None,
+            }
+        out["all_configs"] = allc
+        del step
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(args.config, wl)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

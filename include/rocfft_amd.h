@@ -31,6 +31,33 @@ ROCFFT_EXPORT rocfft_status rocfft_amd_plan_describe(rocfft_result_placement    
                                                      size_t                        text_len,
                                                      size_t*                       work_buffer_bytes);
 
+/*
+ * Per-pass profiling, the counterpart of the reference's profile log layer
+ * (library/src/powX.cpp:817-883 brackets every kernel with hipEvents when
+ * ROCFFT_LAYER has the profile bit).  A plan is a short list of passes, one
+ * kernel launch each.
+ */
+ROCFFT_EXPORT rocfft_status rocfft_amd_plan_get_pass_count(const rocfft_plan plan, size_t* count);
+
+/* Name of pass `index` and the data bytes it reads plus writes (tables excluded). */
+ROCFFT_EXPORT rocfft_status rocfft_amd_plan_get_pass_info(const rocfft_plan plan,
+                                                          size_t            index,
+                                                          char*             name,
+                                                          size_t            name_len,
+                                                          double*           bytes_read_written);
+
+/*
+ * rocfft_execute with every pass bracketed by events on the execution stream;
+ * waits for the stream and writes one duration in milliseconds per pass.
+ * capacity must be at least the pass count.  Not usable during graph capture.
+ */
+ROCFFT_EXPORT rocfft_status rocfft_amd_execute_profile(const rocfft_plan     plan,
+                                                       void*                 in_buffer[],
+                                                       void*                 out_buffer[],
+                                                       rocfft_execution_info info,
+                                                       float*                pass_ms,
+                                                       size_t                capacity);
+
 #ifdef __cplusplus
 }
 #endif

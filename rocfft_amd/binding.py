@@ -85,6 +85,11 @@ _PROTOTYPES = {
     "rocfft_amd_plan_describe": [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_size_t, _c_size_p,
                                  ctypes.c_size_t, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t,
                                  _c_size_p],
+    "rocfft_amd_plan_get_pass_count": [ctypes.c_void_p, _c_size_p],
+    "rocfft_amd_plan_get_pass_info": [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_char_p, ctypes.c_size_t,
+                                      ctypes.POINTER(ctypes.c_double)],
+    "rocfft_amd_execute_profile": [ctypes.c_void_p, _c_void_pp, _c_void_pp, ctypes.c_void_p,
+                                   ctypes.POINTER(ctypes.c_float), ctypes.c_size_t],
 }
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
@@ -255,6 +260,34 @@ class Plan:
 
     def execute(self, in_ptrs, out_ptrs=None, info=None):
         self.lib.check(self.execute_status(in_ptrs, out_ptrs, info), "rocfft_execute")
+
+    def passes(self):
+        """[(name, bytes read + written)] of the plan's kernel launches, in order"""
+        n = ctypes.c_size_t(0)
+        self.lib.check(self.lib.c.rocfft_amd_plan_get_pass_count(self.handle, ctypes.byref(n)),
+                       "rocfft_amd_plan_get_pass_count")
+        out = []
+        for i in range(n.value):
+            name = ctypes.create_string_buffer(256)
+            nbytes = ctypes.c_double(0)
+            self.lib.check(self.lib.c.rocfft_amd_plan_get_pass_info(self.handle, i, name, 256,
+                                                                    ctypes.byref(nbytes)),
+                           "rocfft_amd_plan_get_pass_info")
+            out.append((name.value.decode(), nbytes.value))
+        return out
+
+    def execute_profile(self, in_ptrs, out_ptrs=None, info=None):
+        """like execute, but waits and returns the duration of every pass in milliseconds"""
+        npass = len(self.passes())
+        ms = (ctypes.c_float * max(npass, 1))()
+        ins = (ctypes.c_void_p * 2)(*(list(in_ptrs) + [None])[:2])
+        outs = None
+        if out_ptrs is not None:
+            outs = (ctypes.c_void_p * 2)(*(list(out_ptrs) + [None])[:2])
+        st = self.lib.c.rocfft_amd_execute_profile(self.handle, ins, outs, info.handle if info else None,
+                                                   ms, npass)
+        self.lib.check(st, "rocfft_amd_execute_profile")
+        return [ms[i] for i in range(npass)]
 
     def destroy(self):
         if self.handle:

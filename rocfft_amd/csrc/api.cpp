@@ -311,8 +311,8 @@ rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement plac
     }
 }
 
-rocfft_status rocfft_execute(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
-                             rocfft_execution_info info)
+static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
+                                  rocfft_execution_info info, float* pass_ms)
 {
     if(!plan || !in_buffer || !in_buffer[0])
         return rocfft_status_failure;
@@ -362,7 +362,9 @@ rocfft_status rocfft_execute(const rocfft_plan plan, void* in_buffer[], void* ou
                 own = true;
             }
         }
-        rocfft_status st = run_exec_plan(ep, in, out, work, stream);
+        if(pass_ms && fftrt_stream_capturing(stream))
+            return rocfft_status_failure;
+        rocfft_status st = run_exec_plan(ep, in, out, work, stream, pass_ms);
         if(own)
         {
             fftrt_stream_sync(stream);
@@ -374,6 +376,45 @@ rocfft_status rocfft_execute(const rocfft_plan plan, void* in_buffer[], void* ou
     {
         return rocfft_status_failure;
     }
+}
+
+rocfft_status rocfft_execute(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
+                             rocfft_execution_info info)
+{
+    return execute_impl(plan, in_buffer, out_buffer, info, nullptr);
+}
+
+rocfft_status rocfft_amd_execute_profile(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
+                                         rocfft_execution_info info, float* pass_ms, size_t capacity)
+{
+    if(!plan || !pass_ms || capacity < plan->exec.passes.size())
+        return rocfft_status_invalid_arg_value;
+    return execute_impl(plan, in_buffer, out_buffer, info, pass_ms);
+}
+
+rocfft_status rocfft_amd_plan_get_pass_count(const rocfft_plan plan, size_t* count)
+{
+    if(!plan || !count)
+        return rocfft_status_failure;
+    *count = plan->exec.passes.size();
+    return rocfft_status_success;
+}
+
+rocfft_status rocfft_amd_plan_get_pass_info(const rocfft_plan plan, size_t index, char* name,
+                                            size_t name_len, double* bytes_read_written)
+{
+    if(!plan || index >= plan->exec.passes.size())
+        return rocfft_status_invalid_arg_value;
+    const PassRec& r = plan->exec.passes[index];
+    if(name && name_len)
+    {
+        size_t ncopy = std::min(name_len - 1, r.note.size());
+        memcpy(name, r.note.data(), ncopy);
+        name[ncopy] = 0;
+    }
+    if(bytes_read_written)
+        *bytes_read_written = r.bytes_rw;
+    return rocfft_status_success;
 }
 
 rocfft_status rocfft_plan_destroy(rocfft_plan plan)

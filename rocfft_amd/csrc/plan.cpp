@@ -661,6 +661,31 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     if(s.load_op == FFTK_LOAD_REAL || s.store_op == FFTK_STORE_REAL)
         vec = false;
     rec.vec_ok = vec;
+
+    // data volume of the pass: every element it loads plus every element it stores
+    {
+        double lines   = (double)k.tile_cnt * k.oc[0] * k.oc[1] * k.oc[2];
+        double aux_cnt = 1;
+        if(k.aux_dim == 1)
+            aux_cnt = k.tile_cnt;
+        else if(k.aux_dim >= 2)
+            aux_cnt = k.oc[k.aux_dim - 2];
+        double scalar   = precision ? 8 : 4;
+        double in_elems = lines * std::min(k.n_in, k.n);
+        if(k.load_op == FFTK_LOAD_C2R_PRE)
+            in_elems = lines * (k.n + 1);
+        else if(k.load_op == FFTK_LOAD_HERM_EXPAND)
+            in_elems = lines * (k.n_in / 2 + 1);
+        if((k.flags & FFTK_F_CHIRP_LOAD) && k.chirp_qs)
+            in_elems = lines / aux_cnt * k.blu_n;
+        double out_elems = lines * std::min(k.n_out, k.n);
+        if(k.store_op == FFTK_STORE_R2C_POST)
+            out_elems = lines * (k.n + 1);
+        if((k.flags & FFTK_F_CHIRP_STORE) && k.chirp_qs)
+            out_elems = lines / aux_cnt * k.blu_n;
+        rec.bytes_rw = in_elems * scalar * (k.load_op == FFTK_LOAD_REAL ? 1 : 2)
+                       + out_elems * scalar * (k.store_op == FFTK_STORE_REAL ? 1 : 2);
+    }
     return rec;
 }
 
@@ -1143,6 +1168,12 @@ static void emit_real_step(Builder& b, PassKind kind, uint64_t half, const std::
         rec.src = h;
         rec.dst = z;
     }
+    {
+        double rowsn = 1;
+        for(const Other& o : rows)
+            rowsn *= o.cnt;
+        rec.bytes_rw = rowsn * (2.0 * half + 1) * 2 * (b.precision ? 8 : 4);
+    }
     rec.note = dims_note(kind == PASS_REAL_POST ? "real post-process" : "real pre-process", 2 * half);
     b.plan->passes.push_back(rec);
 }
@@ -1354,8 +1385,20 @@ static bool aligned(const void* p, size_t a)
 }
 
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
-                            void* stream)
+                            void* stream, float* pass_ms)
 {
+    // optional per-pass timing (the reference's profile layer does the same with
+    // hipEvents around every kernel, library/src/powX.cpp:817-883)
+    std::vector<void*> events;
+    if(pass_ms)
+    {
+        events.resize(plan.passes.size() + 1, nullptr);
+        for(void*& e : events)
+            if(fftrt_event_create(&e) != 0)
+                return rocfft_status_failure;
+        fftrt_event_record(events[0], stream);
+    }
+    size_t pass_index = 0;
     const size_t scalar = plan.precision ? 8 : 4;
     char*        tmp    = static_cast<char*>(work);
     char*        blu    = tmp ? tmp + plan.tmp_elems * plan.elem_bytes : nullptr;
@@ -1430,6 +1473,17 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
         }
         if(rc != 0)
             return rocfft_status_failure;
+        ++pass_index;
+        if(pass_ms)
+            fftrt_event_record(events[pass_index], stream);
+    }
+    if(pass_ms)
+    {
+        for(size_t i = 0; i < plan.passes.size(); ++i)
+            if(fftrt_event_elapsed_ms(events[i], events[i + 1], &pass_ms[i]) != 0)
+                pass_ms[i] = -1.0f;
+        for(void* e : events)
+            fftrt_event_destroy(e);
     }
     return rocfft_status_success;
 }

@@ -79,6 +79,7 @@ struct PassRec
     uint32_t              grid   = 0;
     size_t                lds    = 0;
     std::string           note;
+    double                bytes_rw = 0; // data bytes the pass reads plus writes (tables excluded)
     std::vector<TablePtr> tables; // keeps the device tables alive
 };
 
@@ -103,8 +104,10 @@ rocfft_status build_exec_plan(const Problem& prob, ExecPlan& plan, bool dry_run,
 
 // Enqueues every pass on `stream`.  in/out hold one pointer (interleaved, real)
 // or two (planar).  `work` must hold plan.work_bytes() bytes when that is non-zero.
+// When pass_ms is not null every pass is bracketed by events and its duration in
+// milliseconds is written there (the call then waits for the stream).
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
-                            void* stream);
+                            void* stream, float* pass_ms = nullptr);
 
 // drops cached tables that no plan uses any more
 void table_cache_clear();
