@@ -1,0 +1,271 @@
+// fast_core.h -- tile FFT kernel with a compile-time pass schedule.
+//
+// Same tile model as tile_core.h (a workgroup owns W transforms of length N),
+// but length, radices and threads per transform are template parameters, every
+// thread keeps its EPT = max radix elements in registers for the whole kernel,
+// and -- where the lane order matches the fast axis in memory -- the first pass
+// loads straight from global memory into registers and the last pass stores
+// straight from registers, so LDS is only used for the exchanges between passes.
+// When the lane order does not match (row-in/column-out passes) or the fused
+// operation needs partner elements (real pre/post-processing), that side is
+// staged through LDS with tile_load / tile_store of tile_core.h.
+//
+// The reference reaches the same effect with generated kernels
+// ("direct to/from register", library/src/device/generator/stockham_gen_base.h:287-300,
+// :823-913); this is a hand-written template, not generated code.
+#ifndef ROCFFT_AMD_FAST_CORE_H
+#define ROCFFT_AMD_FAST_CORE_H
+
+#include "tile_core.h"
+
+template <int N_, int R0_, int R1_, int R2_, int R3_>
+struct FastCfg
+{
+    static constexpr int N  = N_;
+    static constexpr int R0 = R0_, R1 = R1_, R2 = R2_, R3 = R3_;
+    static constexpr int NP = (R0_ > 1) + (R1_ > 1) + (R2_ > 1) + (R3_ > 1);
+    static constexpr int max2(int a, int b)
+    {
+        return a > b ? a : b;
+    }
+    static constexpr int RMAX = max2(max2(R0_, R1_), max2(R2_, R3_));
+    static constexpr int TPT  = N_ / RMAX; // threads per transform
+    static constexpr int EPT  = RMAX;      // elements per thread
+    static constexpr int radix(int p)
+    {
+        return p == 0 ? R0_ : p == 1 ? R1_ : p == 2 ? R2_ : R3_;
+    }
+    static constexpr int cum(int p)
+    {
+        return p == 0 ? 1 : p == 1 ? R0_ : p == 2 ? R0_ * R1_ : R0_ * R1_ * R2_;
+    }
+    static constexpr int twoff(int p)
+    {
+        // offset of pass p in the stacked twiddle table: sum over 1 <= q < p of cum(q)*(radix(q)-1)
+        return p <= 1 ? 0 : twoff(p - 1) + cum(p - 1) * (radix(p - 1) - 1);
+    }
+    static constexpr int PADSHIFT = 4;
+    static constexpr int PITCH    = (N_ + ((N_ - 1) >> PADSHIFT) + 1) | 1;
+    static_assert(N_ == R0_ * R1_ * R2_ * R3_, "radices must multiply to N");
+    static_assert(RMAX % R0_ == 0 && RMAX % R1_ == 0 && RMAX % R2_ == 0 && RMAX % R3_ == 0,
+                  "every radix must divide the largest one");
+};
+
+template <typename Cfg>
+FFT_DEV uint32_t fk_addr(uint32_t w, uint32_t j)
+{
+    return w * Cfg::PITCH + j + (j >> Cfg::PADSHIFT);
+}
+
+// position of element (butterfly slot s, input k) of pass P held by lane tt
+template <typename Cfg, int P>
+FFT_DEV uint32_t fk_in_pos(uint32_t tt, int s, int k)
+{
+    constexpr int R = Cfg::radix(P);
+    return tt + s * Cfg::TPT + k * (Cfg::N / R);
+}
+
+template <typename Cfg, int P>
+FFT_DEV uint32_t fk_out_pos(uint32_t tt, int s, int k)
+{
+    constexpr int      R = Cfg::radix(P);
+    constexpr uint32_t c = Cfg::cum(P);
+    uint32_t           b = tt + s * Cfg::TPT;
+    return (b / c) * R * c + (b % c) + k * c;
+}
+
+template <typename T, typename Cfg, int P>
+FFT_DEV void fk_read(const typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
+                     typename cplx_of<T>::type* r)
+{
+    constexpr int R = Cfg::radix(P);
+    constexpr int S = Cfg::EPT / R;
+#pragma unroll
+    for(int s = 0; s < S; ++s)
+#pragma unroll
+        for(int k = 0; k < R; ++k)
+            r[s * R + k] = lds[fk_addr<Cfg>(w, fk_in_pos<Cfg, P>(tt, s, k))];
+}
+
+template <typename T, typename Cfg, int P>
+FFT_DEV void fk_write(typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
+                      const typename cplx_of<T>::type* r)
+{
+    constexpr int R = Cfg::radix(P);
+    constexpr int S = Cfg::EPT / R;
+#pragma unroll
+    for(int s = 0; s < S; ++s)
+#pragma unroll
+        for(int k = 0; k < R; ++k)
+            lds[fk_addr<Cfg>(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
+}
+
+template <typename T, typename Cfg, int P>
+FFT_DEV void fk_compute(const fftk_params& p, uint32_t tt, typename cplx_of<T>::type* r)
+{
+    typedef typename cplx_of<T>::type C;
+    constexpr int                     R = Cfg::radix(P);
+    constexpr int                     S = Cfg::EPT / R;
+    constexpr uint32_t                c = Cfg::cum(P);
+#pragma unroll
+    for(int s = 0; s < S; ++s)
+    {
+        if(P > 0)
+        {
+            const C* tw = static_cast<const C*>(p.tw) + Cfg::twoff(P);
+            uint32_t bl = (tt + s * Cfg::TPT) % c;
+#pragma unroll
+            for(int k = 1; k < R; ++k)
+                r[s * R + k] = c_mul(r[s * R + k], tw[(k - 1) * c + bl]);
+        }
+        Butterfly<T, R>::run(r + s * R);
+    }
+}
+
+// all passes on register data; on entry r holds the inputs of pass 0, on exit
+// the outputs of the last pass (element (s,k) at fk_out_pos<last>)
+template <typename T, typename Cfg>
+__device__ __forceinline__ void fk_passes(const fftk_params& p, typename cplx_of<T>::type* lds,
+                                          uint32_t w, uint32_t tt, bool active,
+                                          typename cplx_of<T>::type* r, bool lds_busy)
+{
+#define FK_SYNC() __syncthreads()
+    if(active)
+        fk_compute<T, Cfg, 0>(p, tt, r);
+    if constexpr(Cfg::NP > 1)
+    {
+        if(lds_busy)
+            FK_SYNC();
+        if(active)
+            fk_write<T, Cfg, 0>(lds, w, tt, r);
+        FK_SYNC();
+        if(active)
+        {
+            fk_read<T, Cfg, 1>(lds, w, tt, r);
+            fk_compute<T, Cfg, 1>(p, tt, r);
+        }
+    }
+    if constexpr(Cfg::NP > 2)
+    {
+        FK_SYNC();
+        if(active)
+            fk_write<T, Cfg, 1>(lds, w, tt, r);
+        FK_SYNC();
+        if(active)
+        {
+            fk_read<T, Cfg, 2>(lds, w, tt, r);
+            fk_compute<T, Cfg, 2>(p, tt, r);
+        }
+    }
+    if constexpr(Cfg::NP > 3)
+    {
+        FK_SYNC();
+        if(active)
+            fk_write<T, Cfg, 2>(lds, w, tt, r);
+        FK_SYNC();
+        if(active)
+        {
+            fk_read<T, Cfg, 3>(lds, w, tt, r);
+            fk_compute<T, Cfg, 3>(p, tt, r);
+        }
+    }
+}
+
+template <typename T, typename Cfg, bool VEC>
+__device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cplx_of<T>::type* lds)
+{
+    typedef typename cplx_of<T>::type C;
+    constexpr int                     LAST = Cfg::NP - 1;
+    constexpr int                     RL   = Cfg::radix(LAST);
+    constexpr int                     SL   = Cfg::EPT / RL;
+    constexpr int                     R0   = Cfg::radix(0);
+    constexpr int                     S0   = Cfg::EPT / R0;
+    const uint32_t                    tid  = threadIdx.x;
+    TileCtx<T>                        c;
+    tile_decode<T>(p, blockIdx.x, c);
+    uint32_t w, tt;
+    bool     active = tid < (uint32_t)Cfg::TPT * p.W;
+    if(p.wfast)
+    {
+        w  = tid & (p.W - 1);
+        tt = tid >> p.wshift;
+    }
+    else
+    {
+        tt = tid % (uint32_t)Cfg::TPT;
+        w  = tid / (uint32_t)Cfg::TPT;
+    }
+    C    r[Cfg::EPT];
+    bool lds_busy;
+    if(p.direct_in)
+    {
+        if(active)
+        {
+#pragma unroll
+            for(int s = 0; s < S0; ++s)
+#pragma unroll
+                for(int k = 0; k < R0; ++k)
+                    r[s * R0 + k] = fetch_elem<T, VEC>(p, c, w, fk_in_pos<Cfg, 0>(tt, s, k));
+        }
+        lds_busy = false;
+    }
+    else
+    {
+        tile_load<T, VEC>(p, c, lds, tid);
+        __syncthreads();
+        if(active)
+            fk_read<T, Cfg, 0>(lds, w, tt, r);
+        lds_busy = true;
+    }
+    fk_passes<T, Cfg>(p, lds, w, tt, active, r, lds_busy);
+    if(p.flags & FFTK_F_CONV)
+    {
+        // r holds the forward spectrum: multiply by the stored spectrum, exchange re/im
+        // and run the passes again, which makes the second transform an inverse one
+        uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+        if(Cfg::NP > 1)
+            __syncthreads();
+        if(active)
+        {
+            const bool valid = c.tile0 + w < p.tile_cnt;
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    uint32_t j = fk_out_pos<Cfg, LAST>(tt, s, k);
+                    C        v = r[s * RL + k];
+                    if(valid)
+                        v = c_mul(v, static_cast<const C*>(p.convb)[j + q * p.convb_qs]);
+                    lds[fk_addr<Cfg>(w, j)] = c_swap(v);
+                }
+        }
+        __syncthreads();
+        if(active)
+            fk_read<T, Cfg, 0>(lds, w, tt, r);
+        fk_passes<T, Cfg>(p, lds, w, tt, active, r, true);
+    }
+    if(p.direct_out)
+    {
+        if(active)
+        {
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                    emit_elem<T, VEC>(p, c, w, fk_out_pos<Cfg, LAST>(tt, s, k), r[s * RL + k]);
+        }
+    }
+    else
+    {
+        if(Cfg::NP > 1 || !p.direct_in || (p.flags & FFTK_F_CONV))
+            __syncthreads();
+        if(active)
+            fk_write<T, Cfg, LAST>(lds, w, tt, r);
+        __syncthreads();
+        tile_store<T, VEC>(p, c, lds, tid);
+    }
+}
+#undef FK_SYNC
+
+#endif

@@ -27,6 +27,10 @@ int fftrt_device_sync(void);
 // 1 when `stream` is being captured into a graph
 int fftrt_stream_capturing(void* stream);
 
+// Threads per transform of the compiled-in fast kernel for this exact pass
+// schedule, or 0 when there is none (the generic kernel is used then).
+uint32_t fftrt_fast_tpt(int precision, uint32_t n, const uint32_t* radix, uint32_t nf);
+
 // precision: 0 = float, 1 = double.  vec: 1 when both sides are interleaved
 // complex and can move (re, im) pairs with one access.
 int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,

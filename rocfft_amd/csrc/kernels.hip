@@ -184,10 +184,19 @@ int fftrt_stream_capturing(void* stream)
     return st == hipStreamCaptureStatusActive ? 1 : 0;
 }
 
+int fftrt_launch_fast_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
+                           size_t lds_bytes, void* stream);
+
 int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
                       size_t lds_bytes, void* stream)
 {
     hipStream_t s = (hipStream_t)stream;
+    if(p->fast)
+    {
+        if(p->nthreads == 0 || (p->nthreads & 63) || lds_bytes > MAX_LDS_BYTES || grid == 0)
+            return (int)hipErrorInvalidValue;
+        return fftrt_launch_fast_tile(p, precision, vec, grid, lds_bytes, stream);
+    }
     if(p->nthreads == 0 || p->nthreads > 512 || (p->nthreads & 63) || lds_bytes > MAX_LDS_BYTES
        || grid == 0)
         return (int)hipErrorInvalidValue;

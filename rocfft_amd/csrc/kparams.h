@@ -58,6 +58,9 @@ struct fftk_params
     uint32_t padshift; // LDS index i is stored at i + (i >> padshift)
     uint32_t wfast;    // compute phase: 1 = neighbouring lanes take neighbouring transforms
     uint32_t nthreads;
+    uint32_t fast;       // 1 = a kernel with this exact pass schedule is compiled in: use it
+    uint32_t direct_in;  // fast kernel: first pass loads global memory straight into registers
+    uint32_t direct_out; // fast kernel: last pass stores straight from registers
     uint32_t flags;
     int32_t  dir; // -1 forward, +1 inverse
     uint32_t load_op, store_op;

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -24,6 +25,9 @@ static const uint32_t MAX_THREADS    = 512;
 static const uint32_t PADSHIFT       = 4;
 // a strided ("column") pass wants at least this many bytes contiguous per row of its tile
 static const size_t   COL_RUN_BYTES  = 128;
+
+// ROCFFT_AMD_GENERIC=1 forces the generic tile kernel everywhere (A/B comparisons)
+static const bool g_use_fast = !getenv("ROCFFT_AMD_GENERIC");
 
 struct PlanError : std::runtime_error
 {
@@ -586,8 +590,17 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     k.pitch    = lds_pitch(s.n);
     if(k.T > MAX_THREADS)
         fail("transform too long for one workgroup");
+    // a kernel compiled for exactly this pass schedule, when there is one
+    uint32_t max_threads = MAX_THREADS;
+    uint32_t fast_tpt    = g_use_fast ? fftrt_fast_tpt(precision, k.n, k.radix, k.nf) : 0;
+    if(fast_tpt)
+    {
+        k.fast      = 1;
+        k.T         = fast_tpt;
+        max_threads = 256;
+    }
     size_t   per_tile  = (size_t)k.pitch * esize;
-    uint32_t w_threads = floor_pow2(MAX_THREADS / k.T);
+    uint32_t w_threads = floor_pow2(max_threads / k.T);
     uint32_t w_lds     = per_tile <= LDS_SOFT_BYTES ? floor_pow2(LDS_SOFT_BYTES / per_tile) : 1;
     if(per_tile > LDS_HARD_BYTES)
         fail("transform too long for the LDS of one compute unit");
@@ -611,6 +624,14 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     k.W        = W;
     k.wshift   = log2u(W);
     k.wfast    = W >= 16 ? 1 : 0;
+    if(k.fast)
+    {
+        // lanes follow the fast axis of the input; a side whose fast axis differs, or whose
+        // fused operation needs partner elements, is staged through LDS
+        k.wfast      = k.in_fast_tile;
+        k.direct_in  = s.load_op != FFTK_LOAD_C2R_PRE ? 1 : 0;
+        k.direct_out = (s.store_op != FFTK_STORE_R2C_POST && k.out_fast_tile == k.in_fast_tile) ? 1 : 0;
+    }
     k.nthreads = (k.T * W + 63) / 64 * 64;
     rec.lds    = (size_t)k.pitch * W * esize;
     uint64_t ntile = (k.tile_cnt + W - 1) / W;
@@ -1523,6 +1544,9 @@ std::string ExecPlan::describe() const
               << " lds " << r.lds << " in_fast_" << (k.in_fast_tile ? "tile" : "fft") << " out_fast_"
               << (k.out_fast_tile ? "tile" : "fft") << " flags 0x" << std::hex << k.flags << std::dec
               << " load " << k.load_op << " store " << k.store_op << (r.vec_ok ? " vec" : " scalar");
+            if(k.fast)
+                o << " fast" << (k.direct_in ? " direct_in" : " staged_in")
+                  << (k.direct_out ? " direct_out" : " staged_out");
         }
         else
             o << " half " << r.rp.half << " rows " << r.rp.rows0 << "x" << r.rp.rows1 << "x"

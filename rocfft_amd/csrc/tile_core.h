@@ -110,6 +110,52 @@ FFT_DEV void tile_walk(const fftk_params& p, uint32_t tid, uint32_t jcount, bool
     }
 }
 
+// One logical input element (tile transform w, position j) with the fused input
+// operation applied, ready for the forward butterflies (re/im exchanged when the
+// pass is an inverse transform).  Not used by the C2R pre-processing load.
+template <typename T, bool VEC>
+FFT_DEV typename cplx_of<T>::type
+    fetch_elem(const fftk_params& p, const TileCtx<T>& c, uint32_t w, uint32_t j)
+{
+    typedef typename cplx_of<T>::type C;
+    C                                 v;
+    v.x = 0;
+    v.y = 0;
+    bool     ok  = (c.tile0 + w < p.tile_cnt) && (j < p.n_in);
+    uint32_t idx = 0;
+    if(ok && (p.flags & FFTK_F_CHIRP_LOAD))
+    {
+        uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+        idx        = j * p.chirp_js + q * p.chirp_qs;
+        ok         = idx < p.blu_n;
+    }
+    if(ok)
+    {
+        int64_t base = c.ibase + (int64_t)w * p.w_is;
+        if(p.load_op == FFTK_LOAD_REAL)
+            v.x = static_cast<const T*>(p.in0)[base + (int64_t)j * p.t_is];
+        else if(p.load_op == FFTK_LOAD_HERM_EXPAND)
+        {
+            // logical length n_in; bins above n_in/2 are the conjugate mirror,
+            // imaginary parts of bin 0 and of the Nyquist bin are ignored
+            uint32_t jm = j <= p.n_in / 2 ? j : p.n_in - j;
+            v           = load_elem<T, VEC>(p, base + (int64_t)jm * p.t_is);
+            if(jm != j)
+                v.y = -v.y;
+            if(j == 0 || 2 * j == p.n_in)
+                v.y = 0;
+        }
+        else
+            v = load_elem<T, VEC>(p, base + (int64_t)j * p.t_is);
+        if(p.flags & FFTK_F_CHIRP_LOAD)
+        {
+            C ch = static_cast<const C*>(p.chirp)[idx];
+            v    = (p.flags & FFTK_F_CHIRP_CONJ) ? c_mul(v, ch) : c_mulc(v, ch);
+        }
+    }
+    return p.dir > 0 ? c_swap(v) : v;
+}
+
 template <typename T, bool VEC>
 FFT_DEV void tile_load(const fftk_params&           p,
                        const TileCtx<T>&            c,
@@ -121,42 +167,7 @@ FFT_DEV void tile_load(const fftk_params&           p,
     if(p.load_op != FFTK_LOAD_C2R_PRE)
     {
         tile_walk(p, tid, p.n, p.in_fast_tile != 0, [&](uint32_t w, uint32_t j) {
-            C v;
-            v.x = 0;
-            v.y = 0;
-            bool     ok  = (c.tile0 + w < p.tile_cnt) && (j < p.n_in);
-            uint32_t idx = 0;
-            if(ok && (p.flags & FFTK_F_CHIRP_LOAD))
-            {
-                uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
-                idx        = j * p.chirp_js + q * p.chirp_qs;
-                ok         = idx < p.blu_n;
-            }
-            if(ok)
-            {
-                int64_t base = c.ibase + (int64_t)w * p.w_is;
-                if(p.load_op == FFTK_LOAD_REAL)
-                    v.x = static_cast<const T*>(p.in0)[base + (int64_t)j * p.t_is];
-                else if(p.load_op == FFTK_LOAD_HERM_EXPAND)
-                {
-                    // logical length n_in; bins above n_in/2 are the conjugate mirror,
-                    // imaginary parts of bin 0 and of the Nyquist bin are ignored
-                    uint32_t jm = j <= p.n_in / 2 ? j : p.n_in - j;
-                    v           = load_elem<T, VEC>(p, base + (int64_t)jm * p.t_is);
-                    if(jm != j)
-                        v.y = -v.y;
-                    if(j == 0 || 2 * j == p.n_in)
-                        v.y = 0;
-                }
-                else
-                    v = load_elem<T, VEC>(p, base + (int64_t)j * p.t_is);
-                if(p.flags & FFTK_F_CHIRP_LOAD)
-                {
-                    C ch = static_cast<const C*>(p.chirp)[idx];
-                    v    = (p.flags & FFTK_F_CHIRP_CONJ) ? c_mul(v, ch) : c_mulc(v, ch);
-                }
-            }
-            lds[lds_addr(p, w, j)] = inv ? c_swap(v) : v;
+            lds[lds_addr(p, w, j)] = fetch_elem<T, VEC>(p, c, w, j);
         });
     }
     else
@@ -318,6 +329,46 @@ FFT_DEV typename cplx_of<T>::type large_twiddle(const fftk_params& p, uint32_t u
     return c_mul(lo, hi);
 }
 
+// Writes one logical output element (tile transform w, position j): undoes the
+// re/im exchange of inverse passes, applies the fused output operation, stores.
+// Not used by the R2C post-processing store.
+template <typename T, bool VEC>
+FFT_DEV void emit_elem(const fftk_params& p, const TileCtx<T>& c, uint32_t w, uint32_t j,
+                       typename cplx_of<T>::type v)
+{
+    typedef typename cplx_of<T>::type C;
+    // direction of the transform that produced v
+    const bool inv = (p.flags & FFTK_F_CONV) ? true : (p.dir > 0);
+    if(c.tile0 + w >= p.tile_cnt || j >= p.n_out)
+        return;
+    if(inv)
+        v = c_swap(v);
+    uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+    if(p.flags & FFTK_F_TWIDDLE_STORE)
+    {
+        C t = large_twiddle<T>(p, j * q);
+        v   = inv ? c_mulc(v, t) : c_mul(v, t);
+    }
+    if(p.flags & FFTK_F_CHIRP_STORE)
+    {
+        uint32_t idx = j * p.chirp_js + q * p.chirp_qs;
+        if(idx >= p.blu_n)
+            return;
+        C ch = static_cast<const C*>(p.chirp)[idx];
+        v    = (p.flags & FFTK_F_CHIRP_CONJ) ? c_mul(v, ch) : c_mulc(v, ch);
+    }
+    if(p.flags & FFTK_F_SCALE)
+    {
+        v.x *= (T)p.scale;
+        v.y *= (T)p.scale;
+    }
+    int64_t off = c.obase + (int64_t)j * p.t_os + (int64_t)w * p.w_os;
+    if(p.store_op == FFTK_STORE_REAL)
+        static_cast<T*>(p.out0)[off] = v.x;
+    else
+        store_elem<T, VEC>(p, off, v);
+}
+
 template <typename T, bool VEC>
 FFT_DEV void tile_store(const fftk_params&               p,
                         const TileCtx<T>&                c,
@@ -325,40 +376,10 @@ FFT_DEV void tile_store(const fftk_params&               p,
                         uint32_t                         tid)
 {
     typedef typename cplx_of<T>::type C;
-    // direction of the transform that produced the LDS contents
-    const bool inv = (p.flags & FFTK_F_CONV) ? true : (p.dir > 0);
     if(p.store_op == FFTK_STORE_COMPLEX || p.store_op == FFTK_STORE_REAL)
     {
         tile_walk(p, tid, p.n_out, p.out_fast_tile != 0, [&](uint32_t w, uint32_t j) {
-            if(c.tile0 + w >= p.tile_cnt)
-                return;
-            C v = lds[lds_addr(p, w, j)];
-            if(inv)
-                v = c_swap(v);
-            uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
-            if(p.flags & FFTK_F_TWIDDLE_STORE)
-            {
-                C t = large_twiddle<T>(p, j * q);
-                v   = inv ? c_mulc(v, t) : c_mul(v, t);
-            }
-            if(p.flags & FFTK_F_CHIRP_STORE)
-            {
-                uint32_t idx = j * p.chirp_js + q * p.chirp_qs;
-                if(idx >= p.blu_n)
-                    return;
-                C ch = static_cast<const C*>(p.chirp)[idx];
-                v    = (p.flags & FFTK_F_CHIRP_CONJ) ? c_mul(v, ch) : c_mulc(v, ch);
-            }
-            if(p.flags & FFTK_F_SCALE)
-            {
-                v.x *= (T)p.scale;
-                v.y *= (T)p.scale;
-            }
-            int64_t off = c.obase + (int64_t)j * p.t_os + (int64_t)w * p.w_os;
-            if(p.store_op == FFTK_STORE_REAL)
-                static_cast<T*>(p.out0)[off] = v.x;
-            else
-                store_elem<T, VEC>(p, off, v);
+            emit_elem<T, VEC>(p, c, w, j, lds[lds_addr(p, w, j)]);
         });
     }
     else // FFTK_STORE_R2C_POST

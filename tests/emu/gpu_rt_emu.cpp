@@ -141,6 +141,12 @@ int fftrt_stream_capturing(void*)
     return 0;
 }
 
+// the emulation only has the generic kernel
+uint32_t fftrt_fast_tpt(int, uint32_t, const uint32_t*, uint32_t)
+{
+    return 0;
+}
+
 int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
                       size_t lds_bytes, void*)
 {
