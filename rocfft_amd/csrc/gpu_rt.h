@@ -38,6 +38,10 @@ int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint3
 int fftrt_launch_real_post(const struct fftk_real_params* p, int precision, void* stream);
 int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void* stream);
 
+// 1 when the one-workgroup 32768-point kernel is available in this runtime
+int fftrt_has_big32k(void);
+int fftrt_launch_big32k(const struct fftk_big_params* p, void* stream);
+
 // event timing, used by the optional per-pass profile log
 int fftrt_event_create(void** ev);
 int fftrt_event_destroy(void* ev);

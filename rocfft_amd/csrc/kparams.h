@@ -110,4 +110,20 @@ struct fftk_real_params
     uint32_t    use_scale;
 };
 
+// one-workgroup 32768-point single-precision transform (big_kernels.hip)
+struct fftk_big_params
+{
+    const void* in;
+    void*       out;
+    int64_t     in_line[3], out_line[3]; // strides between transforms, in scalars
+    uint32_t    lines[3];
+    const void* tw;     // stacked twiddles of the radix 32x32x32 schedule
+    const void* half_a; // e^{-2 pi i t/65536}, t in [0, 1024)
+    const void* half_b; // e^{-2 pi i k/64}, k in [0, 32)
+    int32_t     dir;    // complex mode: -1 forward, +1 inverse
+    uint32_t    mode;   // 0 complex, 1 real forward (65536 reals -> 32769 bins), 2 real inverse
+    double      scale;
+    uint32_t    use_scale;
+};
+
 #endif

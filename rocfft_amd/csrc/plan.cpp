@@ -794,6 +794,10 @@ static bool smooth(uint64_t n)
 
 static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t M1, uint64_t M0,
                                    bool conj_chirp);
+static bool     big_eligible(const Builder& b, uint64_t n, int64_t t_is, int64_t t_os,
+                             const std::vector<Other>& others, const IoRef& src, const IoRef& dst);
+static void     emit_big(Builder& b, uint32_t mode, const std::vector<Other>& others, const IoRef& src,
+                         const IoRef& dst, int dir, double scale, bool has_scale);
 
 // One dimension of complex transforms: length n along an axis with scalar strides
 // (t_is, t_os); `others` are the remaining index dimensions.  src and dst may be
@@ -814,6 +818,12 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
             column = true;
     bool plain = ops.load_op == FFTK_LOAD_COMPLEX && ops.store_op == FFTK_STORE_COMPLEX && !ops.n_in
                  && !ops.n_out;
+
+    if(plain && !column && big_eligible(b, n, t_is, t_os, others, src, dst))
+    {
+        emit_big(b, 0, others, src, dst, dir, ops.scale, ops.has_scale);
+        return;
+    }
 
     auto base_spec = [&]() {
         TileSpec s;
@@ -1148,6 +1158,93 @@ static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t 
     return out;
 }
 
+// The one-workgroup 32768-point kernel (big_kernels.hip): single precision, unit stride
+// along the transform on both sides, interleaved data, at most three line dimensions.
+// mode 0: complex (src/dst complex interleaved), 1: real forward (src real pairs, dst
+// Hermitian), 2: real inverse (src Hermitian, dst real pairs).
+static bool big_eligible(const Builder& b, uint64_t n, int64_t t_is, int64_t t_os,
+                         const std::vector<Other>& others, const IoRef& src, const IoRef& dst)
+{
+    if(!g_use_fast || getenv("ROCFFT_AMD_NO_BIG") || b.precision != 0 || n != 32768)
+        return false;
+    if(!fftrt_has_big32k())
+        return false;
+    if(src.planar || dst.planar || src.im_delta != 1 || dst.im_delta != 1 || t_is != 2 || t_os != 2)
+        return false;
+    if((src.off0 & 1) || (dst.off0 & 1))
+        return false;
+    size_t cnt = 0;
+    for(const Other& o : others)
+        if(o.cnt > 1)
+        {
+            ++cnt;
+            if((o.is & 1) || (o.os & 1))
+                return false;
+        }
+    return cnt <= 3;
+}
+
+static void emit_big(Builder& b, uint32_t mode, const std::vector<Other>& others, const IoRef& src,
+                     const IoRef& dst, int dir, double scale, bool has_scale)
+{
+    PassRec rec;
+    rec.kind = PASS_BIG;
+    memset(&rec.kp, 0, sizeof(rec.kp));
+    memset(&rec.rp, 0, sizeof(rec.rp));
+    fftk_big_params& q = rec.bp;
+    memset(&q, 0, sizeof(q));
+    double lines = 1;
+    int    i     = 0;
+    for(int d = 0; d < 3; ++d)
+        q.lines[d] = 1;
+    for(const Other& o : others)
+        if(o.cnt > 1)
+        {
+            q.lines[i]    = o.cnt;
+            q.in_line[i]  = o.is;
+            q.out_line[i] = o.os;
+            lines *= o.cnt;
+            ++i;
+        }
+    q.mode      = mode;
+    q.dir       = dir;
+    q.scale     = scale;
+    q.use_scale = has_scale ? 1 : 0;
+    uint32_t twoff[FFTK_MAX_PASSES];
+    TablePtr tw = stacked_twiddles({32, 32, 32}, 0, b.dry, twoff);
+    TablePtr ha = cached_table("bigA", 0, b.dry, [](HostTable& h) {
+        for(uint64_t t = 0; t < 1024; ++t)
+        {
+            long double c, s;
+            unit_root(t, 65536, c, s);
+            h.push(c, s);
+        }
+    });
+    TablePtr hb = cached_table("bigB", 0, b.dry, [](HostTable& h) {
+        for(uint64_t k = 0; k < 32; ++k)
+        {
+            long double c, s;
+            unit_root(k, 64, c, s);
+            h.push(c, s);
+        }
+    });
+    q.tw     = tw->dptr;
+    q.half_a = ha->dptr;
+    q.half_b = hb->dptr;
+    rec.tables.push_back(tw);
+    rec.tables.push_back(ha);
+    rec.tables.push_back(hb);
+    rec.src  = src;
+    rec.dst  = dst;
+    rec.grid = (uint32_t)lines;
+    rec.lds  = 0;
+    static const char* names[3] = {"one-workgroup fft n=32768", "one-workgroup real forward n=65536",
+                                   "one-workgroup real inverse n=65536"};
+    rec.note     = names[mode];
+    rec.bytes_rw = lines * (mode == 0 ? 2.0 * 32768 * 8 : (65536.0 * 4 + 32769.0 * 8));
+    b.plan->passes.push_back(rec);
+}
+
 // standalone even-length post/pre pass over natural-order rows
 static void emit_real_step(Builder& b, PassKind kind, uint64_t half, const std::vector<Other>& rows,
                            int64_t z_s, const IoRef& z, int64_t h_s, const IoRef& h, double scale,
@@ -1278,7 +1375,9 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                 uint64_t half = n0 / 2;
                 View     rv   = realpair_view(BUF_IN, p.istride, p.idist, p.ioffset, p.rank);
                 auto     oth  = other_axes(rv, hv, p.len, p.rank, p.batch, 0);
-                if(single_kernel_length(half, b.esize))
+                if(big_eligible(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io))
+                    emit_big(b, 1, oth, rv.io, hv.io, -1, p.scale, last0 && p.has_scale);
+                else if(single_kernel_length(half, b.esize))
                 {
                     DimOps ops;
                     ops.store_op = FFTK_STORE_R2C_POST;
@@ -1338,7 +1437,9 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
             uint64_t half = n0 / 2;
             View     rv   = realpair_view(out_buf, p.ostride, p.odist, p.ooffset, p.rank);
             auto     oth  = other_axes(hv, rv, p.len, p.rank, p.batch, 0);
-            if(single_kernel_length(half, b.esize))
+            if(big_eligible(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io))
+                emit_big(b, 2, oth, hv.io, rv.io, +1, p.scale, p.has_scale);
+            else if(single_kernel_length(half, b.esize))
             {
                 DimOps ops;
                 ops.load_op   = FFTK_LOAD_C2R_PRE;
@@ -1462,7 +1563,16 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
         if(!resolve(rec.src, s0, s1) || !resolve(rec.dst, d0, d1))
             return rocfft_status_failure;
         int rc;
-        if(rec.kind == PASS_TILE)
+        if(rec.kind == PASS_BIG)
+        {
+            fftk_big_params q = rec.bp;
+            q.in              = s0;
+            q.out             = d0;
+            if(!aligned(s0, 8) || !aligned(d0, 8))
+                return rocfft_status_failure;
+            rc = fftrt_launch_big32k(&q, stream);
+        }
+        else if(rec.kind == PASS_TILE)
         {
             fftk_params k = rec.kp;
             k.in0         = s0;
@@ -1548,6 +1658,8 @@ std::string ExecPlan::describe() const
                 o << " fast" << (k.direct_in ? " direct_in" : " staged_in")
                   << (k.direct_out ? " direct_out" : " staged_out");
         }
+        else if(r.kind == PASS_BIG)
+            o << " threads 1024 grid " << r.grid << " lds 135296";
         else
             o << " half " << r.rp.half << " rows " << r.rp.rows0 << "x" << r.rp.rows1 << "x"
               << r.rp.rows2;

@@ -56,7 +56,8 @@ enum PassKind
 {
     PASS_TILE      = 0,
     PASS_REAL_POST = 1,
-    PASS_REAL_PRE  = 2
+    PASS_REAL_PRE  = 2,
+    PASS_BIG       = 3 // one-workgroup 32768-point single-precision kernel
 };
 
 // where a pass finds one side of its data: buffer, planar or not, scalar offsets
@@ -74,6 +75,7 @@ struct PassRec
     PassKind              kind = PASS_TILE;
     fftk_params           kp;
     fftk_real_params      rp;
+    fftk_big_params       bp;
     IoRef                 src, dst;
     bool                  vec_ok = false;
     uint32_t              grid   = 0;

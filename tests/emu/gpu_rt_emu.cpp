@@ -176,6 +176,15 @@ int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void*
     return 0;
 }
 
+int fftrt_has_big32k(void)
+{
+    return 0;
+}
+int fftrt_launch_big32k(const struct fftk_big_params*, void*)
+{
+    return 1;
+}
+
 int fftrt_event_create(void** ev)
 {
     *ev = nullptr;
