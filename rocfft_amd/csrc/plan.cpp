@@ -1296,6 +1296,126 @@ static void emit_real_step(Builder& b, PassKind kind, uint64_t half, const std::
     b.plan->passes.push_back(rec);
 }
 
+// A single-pass dimension d followed by a long strided dimension e = d+1 (a "column"
+// dimension too long for one column tile, e.g. the second dimension of a 4096 x 4096
+// transform).  Power-of-two strides between the rows of such an array alias onto the same
+// HBM channel and bank, so reading stride-n0 rows of the user's array runs at a fraction of
+// the streaming rate.  The pass over d therefore writes its rows into the work buffer in
+// permuted order (row n1*n0 + n0' of dimension e goes to slot n0'*n1 + n1) with a padded
+// row pitch: pass A of the split then reads n1 consecutive rows, and pass B reads rows that
+// are a non-power-of-two stride apart before writing the user's output.
+static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t batch, size_t d,
+                             const View& src, const View& out, int dir, const DimOps& last_ops)
+{
+    const size_t e = d + 1;
+    if(e >= rank || getenv("ROCFFT_AMD_NO_STAGED"))
+        return false;
+    const size_t   esize = b.esize;
+    const uint64_t n     = len[e];
+    // dimension e must be strided on both sides and too long for one column tile
+    bool column = false;
+    for(size_t i = 0; i < rank; ++i)
+        if(i != e && len[i] > 1 && (src.stride[i] < src.stride[e] || out.stride[i] < out.stride[e]))
+            column = true;
+    if(!column || !smooth(n) || column_kernel_length(n, esize))
+        return false;
+    uint64_t n1, n0;
+    split_length(n, esize, true, n1, n0);
+    if(n1 == 0)
+        return false;
+    // dimension d must be one plain tile pass
+    bool d_column = false;
+    for(size_t i = 0; i < rank; ++i)
+        if(i != d && len[i] > 1 && (src.stride[i] < src.stride[d]))
+            d_column = true;
+    if(!(d_column ? column_kernel_length(len[d], esize) : single_kernel_length(len[d], esize)))
+        return false;
+    if(src.io.planar || out.io.planar)
+        return false;
+
+    // packed layout of the intermediate array in TMP (scalars)
+    int64_t tstride[4];
+    int64_t run = 2;
+    for(size_t i = 0; i < e; ++i)
+    {
+        tstride[i] = run;
+        run *= (int64_t)len[i];
+    }
+    const int64_t rowS = run + 64; // padded pitch between rows of dimension e
+    const int64_t s_n1 = rowS, s_n0 = (int64_t)n1 * rowS;
+    run                = (int64_t)n * rowS;
+    for(size_t i = e + 1; i < rank; ++i)
+    {
+        tstride[i] = run;
+        run *= (int64_t)len[i];
+    }
+    const int64_t tbatch = run;
+    b.need_tmp((size_t)(tbatch / 2) * batch);
+    IoRef tmp;
+    tmp.buf = BUF_TMP;
+
+    // pass over d: src -> TMP, dimension e split into (n0', n1') with permuted strides
+    {
+        std::vector<Other> oth;
+        for(size_t i = 0; i < rank; ++i)
+        {
+            if(i == d)
+                continue;
+            if(i == e)
+            {
+                oth.push_back({(uint32_t)n0, src.stride[e], s_n0});
+                oth.push_back({(uint32_t)n1, (int64_t)n0 * src.stride[e], s_n1});
+            }
+            else
+                oth.push_back({(uint32_t)len[i], src.stride[i], tstride[i]});
+        }
+        oth.push_back({(uint32_t)batch, src.stride[3], tbatch});
+        emit_dim(b, len[d], src.stride[d], tstride[d], oth, src.io, tmp, dir, DimOps());
+    }
+    TablePtr ltw = large_twiddles(n, b.precision, b.dry);
+    // pass A: n1-point FFT over consecutive rows of TMP, in place, times W_n^{k1 n0'}
+    {
+        TileSpec s;
+        s.dir  = dir;
+        s.n    = (uint32_t)n1;
+        s.t_is = s.t_os = s_n1;
+        s.src = s.dst = tmp;
+        s.others.push_back({(uint32_t)n0, s_n0, s_n0, true});
+        for(size_t i = 0; i < rank; ++i)
+            if(i != e)
+                s.others.push_back({(uint32_t)len[i], tstride[i], tstride[i], false});
+        s.others.push_back({(uint32_t)batch, tbatch, tbatch, false});
+        s.flags |= FFTK_F_TWIDDLE_STORE;
+        s.ltw       = ltw;
+        s.ltw_shift = large_twiddle_shift(n);
+        s.note      = dims_note("staged split A (fft over adjacent rows + twiddle)", n1);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    }
+    // pass B: n0-point FFT over rows n1 apart in TMP, written to the user's rows k1 + n1*k0
+    {
+        TileSpec s;
+        s.dir  = dir;
+        s.n    = (uint32_t)n0;
+        s.t_is = s_n0;
+        s.t_os = (int64_t)n1 * out.stride[e];
+        s.src  = tmp;
+        s.dst  = out.io;
+        s.others.push_back({(uint32_t)n1, s_n1, out.stride[e], false});
+        for(size_t i = 0; i < rank; ++i)
+            if(i != e)
+                s.others.push_back({(uint32_t)len[i], tstride[i], out.stride[i], false});
+        s.others.push_back({(uint32_t)batch, tbatch, out.stride[3], false});
+        if(last_ops.has_scale)
+        {
+            s.flags |= FFTK_F_SCALE;
+            s.scale = last_ops.scale;
+        }
+        s.note = dims_note("staged split B (fft over strided rows, permuted store)", n0);
+        b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------------------
 // whole transforms
 
@@ -1351,7 +1471,13 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
             for(size_t d = 0; d < p.rank; ++d)
             {
                 const View& src = d == 0 ? in : out;
-                DimOps      ops = d + 1 == p.rank ? scale_ops : DimOps();
+                if(emit_dims_staged(b, p.len, p.rank, p.batch, d, src, out, dir,
+                                    d + 2 == p.rank ? scale_ops : DimOps()))
+                {
+                    ++d; // dimensions d and d+1 are done
+                    continue;
+                }
+                DimOps ops = d + 1 == p.rank ? scale_ops : DimOps();
                 emit_dim(b, p.len[d], src.stride[d], out.stride[d],
                          other_axes(src, out, p.len, p.rank, p.batch, d), src.io, out.io, dir, ops);
             }

@@ -199,7 +199,8 @@ def test_pass_lists_of_the_benchmark_configurations(emu):
     st, text, work = emu.describe(B.NOTINPLACE, B.REAL_INVERSE, B.SINGLE, [65536], 4096)
     assert st == 0 and len(passes(text)) <= 3
     st, text, work = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4096, 4096], 8)
-    assert st == 0 and len(passes(text)) <= 3 and work == 8 * 4096 * 4096 * 8
+    # the intermediate of the staged column split is kept with a padded row pitch
+    assert st == 0 and len(passes(text)) <= 3 and 8 * 4096 * 4096 * 8 <= work <= 1.01 * 8 * 4096 * 4096 * 8
     st, text, work = emu.describe(B.NOTINPLACE, B.REAL_FORWARD, B.DOUBLE, [512, 512, 512], 1)
     assert st == 0 and len(passes(text)) == 3 and work == 0
     st, text, work = emu.describe(B.NOTINPLACE, B.REAL_INVERSE, B.DOUBLE, [512, 512, 512], 1)
