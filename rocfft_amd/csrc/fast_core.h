@@ -196,6 +196,76 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
         w  = tid / (uint32_t)Cfg::TPT;
     }
     C    r[Cfg::EPT];
+    if(p.lean)
+    {
+        // Plain interleaved complex data on both sides: every address is a wave-uniform
+        // 64-bit base plus a 32-bit per-lane element offset, and there is no per-element
+        // branching, so the loads of a thread issue back to back.
+        const bool ok  = active && (c.tile0 + w < p.tile_cnt);
+        const bool inv = p.dir > 0;
+        const C*   src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
+        const uint32_t li = tt * p.t_is_c + w * p.w_is_c;
+        if(ok)
+        {
+#pragma unroll
+            for(int s = 0; s < S0; ++s)
+#pragma unroll
+                for(int k = 0; k < R0; ++k)
+                {
+                    const C* pk = src + (uint64_t)(s * Cfg::TPT + k * (Cfg::N / R0)) * p.t_is_c;
+                    r[s * R0 + k] = pk[li];
+                }
+            if(inv)
+            {
+#pragma unroll
+                for(int i = 0; i < Cfg::EPT; ++i)
+                    r[i] = c_swap(r[i]);
+            }
+        }
+        fk_passes<T, Cfg>(p, lds, w, tt, active, r, false);
+        C*             dst = reinterpret_cast<C*>(static_cast<T*>(p.out0) + c.obase);
+        const uint32_t lo  = tt * p.t_os_c + w * p.w_os_c;
+        constexpr int  CL  = Cfg::N / RL; // output (s,k) of the last pass is element tt + s*TPT + k*CL
+        if(ok)
+        {
+            if(inv)
+            {
+#pragma unroll
+                for(int i = 0; i < Cfg::EPT; ++i)
+                    r[i] = c_swap(r[i]);
+            }
+            if(p.flags & FFTK_F_TWIDDLE_STORE)
+            {
+                const uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+#pragma unroll
+                for(int s = 0; s < SL; ++s)
+#pragma unroll
+                    for(int k = 0; k < RL; ++k)
+                    {
+                        C tv         = large_twiddle<T>(p, (tt + s * Cfg::TPT + k * CL) * q);
+                        r[s * RL + k] = inv ? c_mulc(r[s * RL + k], tv) : c_mul(r[s * RL + k], tv);
+                    }
+            }
+            if(p.flags & FFTK_F_SCALE)
+            {
+#pragma unroll
+                for(int i = 0; i < Cfg::EPT; ++i)
+                {
+                    r[i].x *= (T)p.scale;
+                    r[i].y *= (T)p.scale;
+                }
+            }
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
+                    pk[lo] = r[s * RL + k];
+                }
+        }
+        return;
+    }
     bool lds_busy;
     if(p.direct_in)
     {

@@ -61,6 +61,9 @@ struct fftk_params
     uint32_t fast;       // 1 = a kernel with this exact pass schedule is compiled in: use it
     uint32_t direct_in;  // fast kernel: first pass loads global memory straight into registers
     uint32_t direct_out; // fast kernel: last pass stores straight from registers
+    uint32_t lean;       // fast kernel: plain interleaved complex in and out, strides below in
+                         // complex elements fit 32 bits: branch-free addressing path
+    uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
     uint32_t flags;
     int32_t  dir; // -1 forward, +1 inverse
     uint32_t load_op, store_op;

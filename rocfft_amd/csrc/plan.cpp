@@ -682,6 +682,25 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     if(s.load_op == FFTK_LOAD_REAL || s.store_op == FFTK_STORE_REAL)
         vec = false;
     rec.vec_ok = vec;
+    // branch-free addressing path of the fast kernel
+    if(k.fast && vec && k.direct_in && k.direct_out && s.load_op == FFTK_LOAD_COMPLEX
+       && s.store_op == FFTK_STORE_COMPLEX && k.n_in == k.n && k.n_out == k.n
+       && (k.flags & ~(uint32_t)(FFTK_F_TWIDDLE_STORE | FFTK_F_SCALE)) == 0 && k.t_is >= 0 && k.t_os >= 0
+       && k.w_is >= 0 && k.w_os >= 0)
+    {
+        // largest per-lane element offset must fit 32 bits with room to spare
+        uint64_t in_span  = (uint64_t)(k.T - 1) * (uint64_t)(k.t_is / 2) + (uint64_t)(W - 1) * (uint64_t)(k.w_is / 2);
+        uint64_t out_span = (uint64_t)(k.T - 1) * (uint64_t)(k.t_os / 2) + (uint64_t)(W - 1) * (uint64_t)(k.w_os / 2);
+        if(in_span < (1ull << 28) && out_span < (1ull << 28) && (uint64_t)(k.t_is / 2) < (1ull << 31)
+           && (uint64_t)(k.t_os / 2) < (1ull << 31))
+        {
+            rec.lean_ok = true;
+            k.t_is_c    = (uint32_t)(k.t_is / 2);
+            k.t_os_c    = (uint32_t)(k.t_os / 2);
+            k.w_is_c    = (uint32_t)(k.w_is / 2);
+            k.w_os_c    = (uint32_t)(k.w_os / 2);
+        }
+    }
 
     // data volume of the pass: every element it loads plus every element it stores
     {
@@ -1706,6 +1725,7 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             k.out0        = d0;
             k.out1        = d1;
             bool vec = rec.vec_ok && aligned(s0, plan.elem_bytes) && aligned(d0, plan.elem_bytes);
+            k.lean   = (rec.lean_ok && vec) ? 1 : 0;
             rc = fftrt_launch_tile(&k, plan.precision, vec ? 1 : 0, rec.grid, rec.lds, stream);
         }
         else
@@ -1780,6 +1800,8 @@ std::string ExecPlan::describe() const
               << " lds " << r.lds << " in_fast_" << (k.in_fast_tile ? "tile" : "fft") << " out_fast_"
               << (k.out_fast_tile ? "tile" : "fft") << " flags 0x" << std::hex << k.flags << std::dec
               << " load " << k.load_op << " store " << k.store_op << (r.vec_ok ? " vec" : " scalar");
+            if(r.lean_ok)
+                o << " lean";
             if(k.fast)
                 o << " fast" << (k.direct_in ? " direct_in" : " staged_in")
                   << (k.direct_out ? " direct_out" : " staged_out");

@@ -78,6 +78,7 @@ struct PassRec
     fftk_big_params       bp;
     IoRef                 src, dst;
     bool                  vec_ok = false;
+    bool                  lean_ok = false; // eligible for the branch-free addressing path when vec holds
     uint32_t              grid   = 0;
     size_t                lds    = 0;
     std::string           note;
