@@ -171,6 +171,323 @@ __device__ __forceinline__ void fk_passes(const fftk_params& p, typename cplx_of
     }
 }
 
+// Lean path: both sides are interleaved complex arrays whose element offsets inside a
+// tile fit 32 bits.  Every address is a wave-uniform 64-bit base plus a 32-bit per-lane
+// element offset and there is no per-element branching on the operation kind, so the loads
+// of a thread issue back to back.  Covers plain passes, the large twiddle, scaling, the
+// Bluestein chirp on either side, convolution mode, the fused real pre/post-processing and
+// row-in/column-out passes.
+template <typename T, typename Cfg>
+__device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cplx_of<T>::type* lds,
+                                               const TileCtx<T>& c, uint32_t tid, uint32_t w,
+                                               uint32_t tt, bool active)
+{
+    typedef typename cplx_of<T>::type C;
+    constexpr int                     N    = Cfg::N;
+    constexpr int                     LAST = Cfg::NP - 1;
+    constexpr int                     RL   = Cfg::radix(LAST);
+    constexpr int                     SL   = Cfg::EPT / RL;
+    constexpr int                     CL   = N / RL; // output (s,k) of the last pass is element tt + s*TPT + k*CL
+    constexpr int                     R0   = Cfg::radix(0);
+    constexpr int                     S0   = Cfg::EPT / R0;
+    constexpr int                     M0   = N / R0; // input (s,k) of pass 0 is element tt + s*TPT + k*M0
+    const bool                        ok   = active && (c.tile0 + w < p.tile_cnt);
+    const bool                        inv  = p.dir > 0;
+    const C*       src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
+    C*             dst = reinterpret_cast<C*>(static_cast<T*>(p.out0) + c.obase);
+    const uint32_t q   = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+    C              r[Cfg::EPT];
+    bool           lds_busy = false;
+
+    // ---------------------------------------------------------------- load
+    if(p.load_op == FFTK_LOAD_C2R_PRE)
+    {
+        // Hermitian bins -> half-length complex input (library/src/device/kernels/
+        // real2complex_device.h:212-254).  A thread takes the pairs (j, N-j), j = tt + TPT*i < N/2,
+        // writes z_j and z_{N-j} to LDS in natural order; pass 0 then reads from LDS.
+        const C*       htw = static_cast<const C*>(p.half_tw);
+        const uint32_t wo  = w * p.w_is_c;
+        if(ok)
+        {
+#pragma unroll
+            for(int i = 0; i < Cfg::EPT / 2; ++i)
+            {
+                const uint32_t j  = tt + i * Cfg::TPT;
+                const uint32_t jq = N - j;
+                C              a  = src[j * p.t_is_c + wo];
+                C              bq = src[jq * p.t_is_c + wo];
+                C              zj, zq;
+                if(j == 0)
+                {
+                    zj.x = a.x + bq.x;
+                    zj.y = a.x - bq.x;
+                }
+                else
+                {
+                    C t  = htw[j];
+                    C u  = c_add(a, bq);
+                    C v  = c_sub(a, bq);
+                    zj.x = u.x + v.x * t.y - u.y * t.x;
+                    zj.y = v.y + u.y * t.y + v.x * t.x;
+                    zq.x = u.x - v.x * t.y + u.y * t.x;
+                    zq.y = -v.y + u.y * t.y + v.x * t.x;
+                    lds[fk_addr<Cfg>(w, jq)] = c_swap(zq);
+                }
+                lds[fk_addr<Cfg>(w, j)] = c_swap(zj);
+            }
+            if(tt == 0)
+            {
+                C a = src[(N / 2) * p.t_is_c + wo];
+                C z;
+                z.x                         = (T)2 * a.x;
+                z.y                         = (T)-2 * a.y;
+                lds[fk_addr<Cfg>(w, N / 2)] = c_swap(z);
+            }
+        }
+        __syncthreads();
+        if(active)
+            fk_read<T, Cfg, 0>(lds, w, tt, r);
+        lds_busy = true;
+    }
+    else
+    {
+        const uint32_t li = tt * p.t_is_c + w * p.w_is_c;
+        if(ok)
+        {
+            if(p.flags & FFTK_F_CHIRP_LOAD)
+            {
+                const C*   chirp = static_cast<const C*>(p.chirp);
+                const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
+#pragma unroll
+                for(int s = 0; s < S0; ++s)
+#pragma unroll
+                    for(int k = 0; k < R0; ++k)
+                    {
+                        const uint32_t j   = tt + s * Cfg::TPT + k * M0;
+                        const uint32_t idx = j * p.chirp_js + q * p.chirp_qs;
+                        C              v;
+                        v.x = 0;
+                        v.y = 0;
+                        if(idx < p.blu_n)
+                        {
+                            const C* pk = src + (uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c;
+                            C        x  = pk[li];
+                            C        ch = chirp[idx];
+                            v           = cj ? c_mul(x, ch) : c_mulc(x, ch);
+                        }
+                        r[s * R0 + k] = v;
+                    }
+            }
+            else
+            {
+#pragma unroll
+                for(int s = 0; s < S0; ++s)
+#pragma unroll
+                    for(int k = 0; k < R0; ++k)
+                    {
+                        const C* pk = src + (uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c;
+                        r[s * R0 + k] = pk[li];
+                    }
+            }
+            if(inv)
+            {
+#pragma unroll
+                for(int i = 0; i < Cfg::EPT; ++i)
+                    r[i] = c_swap(r[i]);
+            }
+        }
+    }
+
+    // ---------------------------------------------------------------- transform(s)
+    fk_passes<T, Cfg>(p, lds, w, tt, active, r, lds_busy);
+    bool out_inv = inv;
+    if(p.flags & FFTK_F_CONV)
+    {
+        // r holds the forward spectrum: multiply by the stored spectrum, exchange re/im and
+        // run the passes again, which makes the second transform an inverse one
+        if(Cfg::NP > 1 || lds_busy)
+            __syncthreads();
+        if(active)
+        {
+            const C* cb = static_cast<const C*>(p.convb) + (uint64_t)q * p.convb_qs;
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    const uint32_t j = tt + s * Cfg::TPT + k * CL;
+                    C              v = r[s * RL + k];
+                    if(ok)
+                        v = c_mul(v, cb[j]);
+                    lds[fk_addr<Cfg>(w, j)] = c_swap(v);
+                }
+        }
+        __syncthreads();
+        if(active)
+            fk_read<T, Cfg, 0>(lds, w, tt, r);
+        fk_passes<T, Cfg>(p, lds, w, tt, active, r, true);
+        lds_busy = true;
+        out_inv  = true;
+    }
+
+    // ---------------------------------------------------------------- store
+    if(p.store_op == FFTK_STORE_R2C_POST)
+    {
+        // half-length spectrum -> N+1 Hermitian bins (real2complex_device.h:25-103): natural
+        // order through LDS, then a thread produces the pairs (j, N-j)
+        if(Cfg::NP > 1 || lds_busy)
+            __syncthreads();
+        if(active)
+            fk_write<T, Cfg, LAST>(lds, w, tt, r);
+        __syncthreads();
+        if(ok)
+        {
+            const C*       htw = static_cast<const C*>(p.half_tw);
+            const uint32_t wo  = w * p.w_os_c;
+            const T        sc  = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
+#pragma unroll
+            for(int i = 0; i < Cfg::EPT / 2; ++i)
+            {
+                const uint32_t j  = tt + i * Cfg::TPT;
+                const uint32_t jq = N - j;
+                C              zp = lds[fk_addr<Cfg>(w, j)];
+                C              o0, o1;
+                if(j == 0)
+                {
+                    o0.x = zp.x + zp.y;
+                    o0.y = 0;
+                    o1.x = zp.x - zp.y;
+                    o1.y = 0;
+                }
+                else
+                {
+                    C zq = lds[fk_addr<Cfg>(w, jq)];
+                    C t  = htw[j];
+                    C u, v;
+                    u.x  = (T)0.5 * (zp.x + zq.x);
+                    u.y  = (T)0.5 * (zp.y + zq.y);
+                    v.x  = (T)0.5 * (zp.x - zq.x);
+                    v.y  = (T)0.5 * (zp.y - zq.y);
+                    o0.x = u.x + v.x * t.y + u.y * t.x;
+                    o0.y = v.y + u.y * t.y - v.x * t.x;
+                    o1.x = u.x - v.x * t.y - u.y * t.x;
+                    o1.y = -v.y + u.y * t.y - v.x * t.x;
+                }
+                o0.x *= sc;
+                o0.y *= sc;
+                o1.x *= sc;
+                o1.y *= sc;
+                dst[j * p.t_os_c + wo]  = o0;
+                dst[jq * p.t_os_c + wo] = o1;
+            }
+            if(tt == 0)
+            {
+                C z = lds[fk_addr<Cfg>(w, N / 2)];
+                C o;
+                o.x                            = z.x * sc;
+                o.y                            = -z.y * sc;
+                dst[(N / 2) * p.t_os_c + wo] = o;
+            }
+        }
+        return;
+    }
+
+    uint32_t ow = w, ot = tt;
+    bool     ook = ok;
+    if(!p.direct_out)
+    {
+        // the store runs along the other axis than the load did: through LDS in natural
+        // order, then re-read with the lanes running along the tile dimension (or along the
+        // transform) so that the global stores coalesce
+        if(Cfg::NP > 1 || lds_busy)
+            __syncthreads();
+        if(active)
+            fk_write<T, Cfg, LAST>(lds, w, tt, r);
+        __syncthreads();
+        if(p.wfast)
+        {
+            ot = tid % (uint32_t)Cfg::TPT;
+            ow = tid / (uint32_t)Cfg::TPT;
+        }
+        else
+        {
+            ow = tid & (p.W - 1);
+            ot = tid >> p.wshift;
+        }
+        ook = active && (c.tile0 + ow < p.tile_cnt);
+        if(active)
+        {
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                    r[s * RL + k] = lds[fk_addr<Cfg>(ow, ot + s * Cfg::TPT + k * CL)];
+        }
+    }
+    const uint32_t oq = p.aux_dim == 1 ? c.tile0 + ow : c.q_block;
+    const uint32_t lo = ot * p.t_os_c + ow * p.w_os_c;
+    if(ook)
+    {
+        if(out_inv)
+        {
+#pragma unroll
+            for(int i = 0; i < Cfg::EPT; ++i)
+                r[i] = c_swap(r[i]);
+        }
+        if(p.flags & FFTK_F_TWIDDLE_STORE)
+        {
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    C tv          = large_twiddle<T>(p, (ot + s * Cfg::TPT + k * CL) * oq);
+                    r[s * RL + k] = out_inv ? c_mulc(r[s * RL + k], tv) : c_mul(r[s * RL + k], tv);
+                }
+        }
+        if(p.flags & FFTK_F_SCALE)
+        {
+#pragma unroll
+            for(int i = 0; i < Cfg::EPT; ++i)
+            {
+                r[i].x *= (T)p.scale;
+                r[i].y *= (T)p.scale;
+            }
+        }
+        if(p.flags & FFTK_F_CHIRP_STORE)
+        {
+            const C*   chirp = static_cast<const C*>(p.chirp);
+            const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    const uint32_t j   = ot + s * Cfg::TPT + k * CL;
+                    const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
+                    if(idx < p.blu_n && j < p.n_out)
+                    {
+                        C  ch  = chirp[idx];
+                        C  v   = cj ? c_mul(r[s * RL + k], ch) : c_mulc(r[s * RL + k], ch);
+                        C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
+                        pk[lo] = v;
+                    }
+                }
+        }
+        else
+        {
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
+                    pk[lo] = r[s * RL + k];
+                }
+        }
+    }
+}
+
 template <typename T, typename Cfg, bool VEC>
 __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cplx_of<T>::type* lds)
 {
@@ -195,77 +512,12 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
         tt = tid % (uint32_t)Cfg::TPT;
         w  = tid / (uint32_t)Cfg::TPT;
     }
-    C    r[Cfg::EPT];
-    if(p.lean)
+    if(VEC && p.lean)
     {
-        // Plain interleaved complex data on both sides: every address is a wave-uniform
-        // 64-bit base plus a 32-bit per-lane element offset, and there is no per-element
-        // branching, so the loads of a thread issue back to back.
-        const bool ok  = active && (c.tile0 + w < p.tile_cnt);
-        const bool inv = p.dir > 0;
-        const C*   src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
-        const uint32_t li = tt * p.t_is_c + w * p.w_is_c;
-        if(ok)
-        {
-#pragma unroll
-            for(int s = 0; s < S0; ++s)
-#pragma unroll
-                for(int k = 0; k < R0; ++k)
-                {
-                    const C* pk = src + (uint64_t)(s * Cfg::TPT + k * (Cfg::N / R0)) * p.t_is_c;
-                    r[s * R0 + k] = pk[li];
-                }
-            if(inv)
-            {
-#pragma unroll
-                for(int i = 0; i < Cfg::EPT; ++i)
-                    r[i] = c_swap(r[i]);
-            }
-        }
-        fk_passes<T, Cfg>(p, lds, w, tt, active, r, false);
-        C*             dst = reinterpret_cast<C*>(static_cast<T*>(p.out0) + c.obase);
-        const uint32_t lo  = tt * p.t_os_c + w * p.w_os_c;
-        constexpr int  CL  = Cfg::N / RL; // output (s,k) of the last pass is element tt + s*TPT + k*CL
-        if(ok)
-        {
-            if(inv)
-            {
-#pragma unroll
-                for(int i = 0; i < Cfg::EPT; ++i)
-                    r[i] = c_swap(r[i]);
-            }
-            if(p.flags & FFTK_F_TWIDDLE_STORE)
-            {
-                const uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
-#pragma unroll
-                for(int s = 0; s < SL; ++s)
-#pragma unroll
-                    for(int k = 0; k < RL; ++k)
-                    {
-                        C tv         = large_twiddle<T>(p, (tt + s * Cfg::TPT + k * CL) * q);
-                        r[s * RL + k] = inv ? c_mulc(r[s * RL + k], tv) : c_mul(r[s * RL + k], tv);
-                    }
-            }
-            if(p.flags & FFTK_F_SCALE)
-            {
-#pragma unroll
-                for(int i = 0; i < Cfg::EPT; ++i)
-                {
-                    r[i].x *= (T)p.scale;
-                    r[i].y *= (T)p.scale;
-                }
-            }
-#pragma unroll
-            for(int s = 0; s < SL; ++s)
-#pragma unroll
-                for(int k = 0; k < RL; ++k)
-                {
-                    C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
-                    pk[lo] = r[s * RL + k];
-                }
-        }
+        fast_tile_lean<T, Cfg>(p, lds, c, tid, w, tt, active);
         return;
     }
+    C    r[Cfg::EPT];
     bool lds_busy;
     if(p.direct_in)
     {

@@ -682,23 +682,38 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     if(s.load_op == FFTK_LOAD_REAL || s.store_op == FFTK_STORE_REAL)
         vec = false;
     rec.vec_ok = vec;
-    // branch-free addressing path of the fast kernel
-    if(k.fast && vec && k.direct_in && k.direct_out && s.load_op == FFTK_LOAD_COMPLEX
-       && s.store_op == FFTK_STORE_COMPLEX && k.n_in == k.n && k.n_out == k.n
-       && (k.flags & ~(uint32_t)(FFTK_F_TWIDDLE_STORE | FFTK_F_SCALE)) == 0 && k.t_is >= 0 && k.t_os >= 0
-       && k.w_is >= 0 && k.w_os >= 0)
+    // branch-free addressing path of the fast kernel: interleaved complex on both sides
+    // (real pairs with unit real stride count), element offsets inside a tile fit 32 bits
     {
-        // largest per-lane element offset must fit 32 bits with room to spare
-        uint64_t in_span  = (uint64_t)(k.T - 1) * (uint64_t)(k.t_is / 2) + (uint64_t)(W - 1) * (uint64_t)(k.w_is / 2);
-        uint64_t out_span = (uint64_t)(k.T - 1) * (uint64_t)(k.t_os / 2) + (uint64_t)(W - 1) * (uint64_t)(k.w_os / 2);
-        if(in_span < (1ull << 28) && out_span < (1ull << 28) && (uint64_t)(k.t_is / 2) < (1ull << 31)
-           && (uint64_t)(k.t_os / 2) < (1ull << 31))
+        const uint32_t lean_flags = FFTK_F_TWIDDLE_STORE | FFTK_F_SCALE | FFTK_F_CHIRP_LOAD
+                                    | FFTK_F_CHIRP_STORE | FFTK_F_CHIRP_CONJ | FFTK_F_CONV;
+        bool ops_ok = (s.load_op == FFTK_LOAD_COMPLEX || s.load_op == FFTK_LOAD_C2R_PRE)
+                      && (s.store_op == FFTK_STORE_COMPLEX || s.store_op == FFTK_STORE_R2C_POST)
+                      && (k.flags & ~lean_flags) == 0;
+        // short inputs/outputs are only expressed through the chirp index test
+        if(k.n_in != k.n && !((k.flags & FFTK_F_CHIRP_LOAD) && k.chirp_js == 1 && k.chirp_qs == 0
+                              && k.n_in == k.blu_n))
+            ops_ok = false;
+        if(k.n_out != k.n && !(k.flags & FFTK_F_CHIRP_STORE))
+            ops_ok = false;
+        if(s.load_op == FFTK_LOAD_C2R_PRE && (k.flags & (FFTK_F_CHIRP_LOAD | FFTK_F_CONV)))
+            ops_ok = false;
+        if(s.store_op == FFTK_STORE_R2C_POST && (k.flags & (FFTK_F_CHIRP_STORE | FFTK_F_TWIDDLE_STORE)))
+            ops_ok = false;
+        if((s.load_op == FFTK_LOAD_C2R_PRE || s.store_op == FFTK_STORE_R2C_POST) && (k.n & 1))
+            ops_ok = false;
+        if(k.fast && vec && ops_ok && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
         {
-            rec.lean_ok = true;
-            k.t_is_c    = (uint32_t)(k.t_is / 2);
-            k.t_os_c    = (uint32_t)(k.t_os / 2);
-            k.w_is_c    = (uint32_t)(k.w_is / 2);
-            k.w_os_c    = (uint32_t)(k.w_os / 2);
+            uint64_t in_span  = (uint64_t)(k.n + 1) * (uint64_t)(k.t_is / 2) + (uint64_t)W * (uint64_t)(k.w_is / 2);
+            uint64_t out_span = (uint64_t)(k.n + 1) * (uint64_t)(k.t_os / 2) + (uint64_t)W * (uint64_t)(k.w_os / 2);
+            if(in_span < (1ull << 28) && out_span < (1ull << 28))
+            {
+                rec.lean_ok = true;
+                k.t_is_c    = (uint32_t)(k.t_is / 2);
+                k.t_os_c    = (uint32_t)(k.t_os / 2);
+                k.w_is_c    = (uint32_t)(k.w_is / 2);
+                k.w_os_c    = (uint32_t)(k.w_os / 2);
+            }
         }
     }
 
