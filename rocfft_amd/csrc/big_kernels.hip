@@ -104,10 +104,11 @@ __device__ __forceinline__ constexpr int big_slot_index(int s)
     return 8 * (s & 3) + (s >> 2);
 }
 
-__device__ __forceinline__ uint32_t big_pad(uint32_t i)
-{
-    return i + (i >> 5);
-}
+// Padded LDS index of scalar i is i + (i >> 5) (one pad word per 32).  With t < 1024 and
+// k < 32 the three access patterns reduce to a per-thread base plus a compile-time offset:
+//   i = 32 t + k              -> 33 t + k
+//   i = t + 1024 k            -> t + (t >> 5) + 1056 k
+//   i = (t/32) 1024 + t%32 + 32 k -> (t >> 5) 1056 + (t & 31) + 33 k
 
 // r[k] *= w^k for k = 1..31 with w^1..w^7 and w^8, w^16, w^24 read from the stacked
 // table of the pass (entry (k-1)*c + bl) and the rest formed as w^(8a) * w^b
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
             float2         xa = hx[j];
             float2         xb = hx[BIG_L - j];
             float2         zj, zq;
-            if(j == 0)
+            if(k == 0 && t == 0)
             {
                 zj.x = xa.x + xb.x;
                 zj.y = xa.x - xb.x;
@@ -216,45 +217,52 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
         __syncthreads();
     }
 
+    const uint32_t w1base = 33 * t;
+    const uint32_t rbase  = t + (t >> 5);
+    const uint32_t w2base = (t >> 5) * 1056 + (t & 31);
     // ---- pass 0 (outputs in slot order: slot s holds output big_slot_index(s))
     Butterfly32<float>::run(r);
     // exchange 1: write 32 t + k_out, read t + 1024 k
 #pragma unroll
     for(int s = 0; s < BIG_EPT; ++s)
-        lds[big_pad(32 * t + big_slot_index(s))] = r[s].x;
+        lds[w1base + big_slot_index(s)] = r[s].x;
     __syncthreads();
 #pragma unroll
     for(int k = 0; k < BIG_EPT; ++k)
-        r[k].x = lds[big_pad(t + 1024 * k)];
+        r[k].x = lds[rbase + 1056 * k];
     __syncthreads();
 #pragma unroll
     for(int s = 0; s < BIG_EPT; ++s)
-        lds[big_pad(32 * t + big_slot_index(s))] = r[s].y;
+        lds[w1base + big_slot_index(s)] = r[s].y;
     __syncthreads();
 #pragma unroll
     for(int k = 0; k < BIG_EPT; ++k)
-        r[k].y = lds[big_pad(t + 1024 * k)];
+        r[k].y = lds[rbase + 1056 * k];
     // ---- pass 1 (cumulative height 32)
-    big_twiddle(r, tw, 32u, t & 31u);
+    {
+        const uint32_t bl = t & 31u;
+#pragma unroll
+        for(int k = 1; k < BIG_EPT; ++k)
+            r[k] = c_mul(r[k], tw[(k - 1) * 32 + bl]);
+    }
     Butterfly32<float>::run(r);
     __syncthreads();
     // exchange 2: write (t/32)*1024 + (t%32) + 32 k_out, read t + 1024 k
-    const uint32_t wbase = (t >> 5) * 1024 + (t & 31);
 #pragma unroll
     for(int s = 0; s < BIG_EPT; ++s)
-        lds[big_pad(wbase + 32 * big_slot_index(s))] = r[s].x;
+        lds[w2base + 33 * big_slot_index(s)] = r[s].x;
     __syncthreads();
 #pragma unroll
     for(int k = 0; k < BIG_EPT; ++k)
-        r[k].x = lds[big_pad(t + 1024 * k)];
+        r[k].x = lds[rbase + 1056 * k];
     __syncthreads();
 #pragma unroll
     for(int s = 0; s < BIG_EPT; ++s)
-        lds[big_pad(wbase + 32 * big_slot_index(s))] = r[s].y;
+        lds[w2base + 33 * big_slot_index(s)] = r[s].y;
     __syncthreads();
 #pragma unroll
     for(int k = 0; k < BIG_EPT; ++k)
-        r[k].y = lds[big_pad(t + 1024 * k)];
+        r[k].y = lds[rbase + 1056 * k];
     // ---- pass 2 (cumulative height 1024); stacked offset of pass 2 is 31*32
     big_twiddle(r, tw + 31 * 32, 1024u, t);
     Butterfly32<float>::run(r);
@@ -307,7 +315,7 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
         const uint32_t j  = t + 1024 * k;
         float2         zp = r[s];
         float2         o0, o1;
-        if(j == 0)
+        if(k == 0 && t == 0)
         {
             o0.x = zp.x + zp.y;
             o0.y = 0.0f;
