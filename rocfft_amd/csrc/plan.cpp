@@ -28,6 +28,8 @@ static const size_t   COL_RUN_BYTES  = 128;
 
 // ROCFFT_AMD_GENERIC=1 forces the generic tile kernel everywhere (A/B comparisons)
 static const bool g_use_fast = !getenv("ROCFFT_AMD_GENERIC");
+// ROCFFT_AMD_NO_XCD_REMAP=1 keeps the hardware's round-robin workgroup order (A/B comparisons)
+static const bool g_xcd_remap = !getenv("ROCFFT_AMD_NO_XCD_REMAP");
 
 struct PlanError : std::runtime_error
 {
@@ -639,6 +641,14 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     if(grid == 0 || grid >= (1ull << 31))
         fail("grid too large");
     rec.grid = (uint32_t)grid;
+    k.grid      = rec.grid;
+    // Neighbouring column tiles share 128-byte lines when the rows of the array are not
+    // line-aligned; then each XCD should own a contiguous range of tiles.
+    {
+        const int64_t line  = 128 / (precision ? 8 : 4); // scalars per 128 bytes
+        const bool    split = (k.in_fast_tile && (k.t_is % line)) || (k.out_fast_tile && (k.t_os % line));
+        k.xcd_remap         = (g_xcd_remap && column && split && rec.grid >= 64) ? 1 : 0;
+    }
 
     k.flags    = s.flags;
     k.dir      = s.dir;

@@ -33,6 +33,15 @@ struct TileCtx
 template <typename T>
 FFT_DEV void tile_decode(const fftk_params& p, uint32_t bid, TileCtx<T>& c)
 {
+    if(p.xcd_remap)
+    {
+        // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Renumber so
+        // that every XCD works through one contiguous range of tiles: neighbouring tiles,
+        // which share cache lines and DRAM pages, then meet in the same L2 at the same time.
+        const uint32_t grid = p.grid, xcd = bid & 7u, idx = bid >> 3;
+        const uint32_t qd = grid >> 3, rm = grid & 7u;
+        bid = xcd * qd + (xcd < rm ? xcd : rm) + idx;
+    }
     uint32_t ntile = (p.tile_cnt + p.W - 1) >> p.wshift;
     uint32_t tb    = bid % ntile;
     bid /= ntile;
