@@ -256,8 +256,23 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         {
             if(p.flags & FFTK_F_CHIRP_LOAD)
             {
+                // samples beyond the signal read as zero; their loads are redirected to the
+                // first sample instead of being skipped, so that all loads stay in flight
                 const C*   chirp = static_cast<const C*>(p.chirp);
                 const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
+                C          ch[Cfg::EPT];
+#pragma unroll
+                for(int s = 0; s < S0; ++s)
+#pragma unroll
+                    for(int k = 0; k < R0; ++k)
+                    {
+                        const uint32_t j     = tt + s * Cfg::TPT + k * M0;
+                        const uint32_t idx   = j * p.chirp_js + q * p.chirp_qs;
+                        const bool     valid = idx < p.blu_n;
+                        const uint32_t off   = valid ? j * p.t_is_c + w * p.w_is_c : 0u;
+                        r[s * R0 + k]        = src[off];
+                        ch[s * R0 + k]       = chirp[valid ? idx : 0u];
+                    }
 #pragma unroll
                 for(int s = 0; s < S0; ++s)
 #pragma unroll
@@ -265,15 +280,12 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     {
                         const uint32_t j   = tt + s * Cfg::TPT + k * M0;
                         const uint32_t idx = j * p.chirp_js + q * p.chirp_qs;
-                        C              v;
-                        v.x = 0;
-                        v.y = 0;
-                        if(idx < p.blu_n)
+                        C              x   = r[s * R0 + k];
+                        C v = cj ? c_mul(x, ch[s * R0 + k]) : c_mulc(x, ch[s * R0 + k]);
+                        if(idx >= p.blu_n)
                         {
-                            const C* pk = src + (uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c;
-                            C        x  = pk[li];
-                            C        ch = chirp[idx];
-                            v           = cj ? c_mul(x, ch) : c_mulc(x, ch);
+                            v.x = 0;
+                            v.y = 0;
                         }
                         r[s * R0 + k] = v;
                     }
@@ -458,6 +470,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         {
             const C*   chirp = static_cast<const C*>(p.chirp);
             const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
+            C          ch[Cfg::EPT];
 #pragma unroll
             for(int s = 0; s < SL; ++s)
 #pragma unroll
@@ -465,10 +478,18 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 {
                     const uint32_t j   = ot + s * Cfg::TPT + k * CL;
                     const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
+                    ch[s * RL + k]     = chirp[idx < p.blu_n ? idx : 0u];
+                }
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    const uint32_t j   = ot + s * Cfg::TPT + k * CL;
+                    const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
+                    C v = cj ? c_mul(r[s * RL + k], ch[s * RL + k]) : c_mulc(r[s * RL + k], ch[s * RL + k]);
                     if(idx < p.blu_n && j < p.n_out)
                     {
-                        C  ch  = chirp[idx];
-                        C  v   = cj ? c_mul(r[s * RL + k], ch) : c_mulc(r[s * RL + k], ch);
                         C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
                         pk[lo] = v;
                     }

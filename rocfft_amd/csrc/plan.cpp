@@ -1035,15 +1035,18 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         fail("internal: Bluestein split of a short length");
     TablePtr bs  = bluestein_spectrum(b, N, M, M1, M0, conj_chirp);
     TablePtr ltw = large_twiddles(M, b.precision, b.dry);
-    b.need_blu(lines * M);
-    std::vector<int64_t> pk = packed_strides(M);
+    // rows of the padded signals get a pitch that is not a power of two, so that the strided
+    // column passes do not hammer one HBM channel
+    const int64_t rowp = (int64_t)M0 + 16; // complex elements
+    b.need_blu(lines * M1 * (uint64_t)rowp);
+    std::vector<int64_t> pk = packed_strides(M1 * (uint64_t)rowp);
     {
         // Z1: chirp multiply + zero pad fused into the load of the column FFT over n1
         TileSpec s = base_spec();
         s.dir      = -1;
         s.n        = (uint32_t)M1;
         s.t_is     = (int64_t)M0 * t_is;
-        s.t_os     = (int64_t)M0 * 2;
+        s.t_os     = rowp * 2;
         s.src      = src;
         s.dst      = blu;
         s.others.push_back({(uint32_t)M0, t_is, 2, true});
@@ -1067,7 +1070,7 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         s.n        = (uint32_t)M0;
         s.t_is = s.t_os = 2;
         s.src = s.dst = blu;
-        s.others.push_back({(uint32_t)M1, (int64_t)M0 * 2, (int64_t)M0 * 2, true});
+        s.others.push_back({(uint32_t)M1, rowp * 2, rowp * 2, true});
         add_others(s, false, false, pk);
         s.flags |= FFTK_F_CONV | FFTK_F_TWIDDLE_STORE;
         s.convb     = bs;
@@ -1082,7 +1085,7 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         TileSpec s = base_spec();
         s.dir      = +1;
         s.n        = (uint32_t)M1;
-        s.t_is     = (int64_t)M0 * 2;
+        s.t_is     = rowp * 2;
         s.t_os     = (int64_t)M0 * t_os;
         s.src      = blu;
         s.dst      = dst;

@@ -207,7 +207,8 @@ def test_pass_lists_of_the_benchmark_configurations(emu):
     assert st == 0 and len(passes(text)) == 3 and work == 0
     st, text, work = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.DOUBLE, [1000003], 16)
     assert st == 0 and len(passes(text)) == 3 and "bluestein" in text
-    assert work == 16 * 2 ** 21 * 16
+    # 16 zero-padded signals of 2^21 points, rows of 4096 kept at a padded pitch
+    assert 16 * 2 ** 21 * 16 <= work <= 1.01 * 16 * 2 ** 21 * 16
 
 
 def test_every_tile_fits_the_hardware(emu):
