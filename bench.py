@@ -232,6 +232,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default 2)")
     ap.add_argument("--no-extras", action="store_true", help="skip all_configs and the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB) ten times: "
+                         "the known-size kernel the rocprofv3 FETCH_SIZE/WRITE_SIZE counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives one GPU; --gpus %d is not supported "
@@ -246,6 +249,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU", file=sys.stderr)
         sys.exit(1)
+    if args.calibrate_copy:
+        n = 1 << 28  # float32 elements = 1 GiB
+        src = torch.rand(n, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch.mul(src, 1.0, out=dst), float32", "bytes_read": 4 * n,
+                          "bytes_written": 4 * n, "launches": 10}))
+        return
     rf.library()  # raises if the HIP library is not built
     stream_ptr = torch.cuda.current_stream().cuda_stream
     wls = workloads()

@@ -509,7 +509,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     }
 }
 
-template <typename T, typename Cfg, bool VEC>
+template <typename T, typename Cfg, bool VEC, bool LEAN>
 __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cplx_of<T>::type* lds)
 {
     typedef typename cplx_of<T>::type C;
@@ -533,7 +533,7 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
         tt = tid % (uint32_t)Cfg::TPT;
         w  = tid / (uint32_t)Cfg::TPT;
     }
-    if(VEC && p.lean)
+    if constexpr(LEAN)
     {
         fast_tile_lean<T, Cfg>(p, lds, c, tid, w, tt, active);
         return;

@@ -8,20 +8,22 @@
 namespace
 {
 
-template <typename T, typename Cfg, bool VEC>
+// MODE 0: scalar accesses, every fused operation; 1: vector accesses, every fused operation;
+// 2: the lean path (vector accesses, interleaved complex on both sides)
+template <typename T, typename Cfg, int MODE>
 __global__ __launch_bounds__(256) void fast_tile_kernel(const fftk_params p)
 {
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
-    fast_tile_body<T, Cfg, VEC>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE == 2>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 typedef int (*fast_launch_fn)(const fftk_params*, uint32_t, size_t, hipStream_t);
 
-template <typename T, typename Cfg, bool VEC>
+template <typename T, typename Cfg, int MODE>
 int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, hipStream_t stream)
 {
-    auto kernel = fast_tile_kernel<T, Cfg, VEC>;
+    auto kernel = fast_tile_kernel<T, Cfg, MODE>;
     if(lds_bytes > 64 * 1024)
     {
         static std::once_flag once[16];
@@ -45,14 +47,13 @@ struct FastEntry
     uint32_t       n;
     uint32_t       radix[4];
     uint32_t       tpt;
-    fast_launch_fn vec, scalar;
+    fast_launch_fn lean, vec, scalar;
 };
 
-#define FAST_BOTH(N, A, B, C, D)                                                              \
-    {0, N, {A, B, C, D}, FastCfg<N, A, B, C, D>::TPT, &launch_fast<float, FastCfg<N, A, B, C, D>, true>, \
-     &launch_fast<float, FastCfg<N, A, B, C, D>, false>},                                     \
-    {1, N, {A, B, C, D}, FastCfg<N, A, B, C, D>::TPT, &launch_fast<double, FastCfg<N, A, B, C, D>, true>, \
-     &launch_fast<double, FastCfg<N, A, B, C, D>, false>},
+#define FAST_ONE(T, P, N, A, B, C, D)                                                              \
+    {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D>, 2>,  \
+     &launch_fast<T, FastCfg<N, A, B, C, D>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D>, 0>},
+#define FAST_BOTH(N, A, B, C, D) FAST_ONE(float, 0, N, A, B, C, D) FAST_ONE(double, 1, N, A, B, C, D)
 
 // the schedules the planner's factorisation produces for powers of two
 const FastEntry g_fast[] = {
@@ -102,5 +103,6 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
     const FastEntry* e = find_fast(precision, p->n, p->radix, p->nf);
     if(!e || p->T != e->tpt || p->nthreads > 256 || p->padshift != 4)
         return (int)hipErrorInvalidValue;
-    return (vec ? e->vec : e->scalar)(p, grid, lds_bytes, (hipStream_t)stream);
+    fast_launch_fn fn = (vec && p->lean) ? e->lean : vec ? e->vec : e->scalar;
+    return fn(p, grid, lds_bytes, (hipStream_t)stream);
 }

@@ -54,7 +54,8 @@ FFT_DEV void tile_decode(const fftk_params& p, uint32_t bid, TileCtx<T>& c)
               + (int64_t)c.oi[2] * p.o_is[2];
     c.obase = (int64_t)c.tile0 * p.w_os + (int64_t)c.oi[0] * p.o_os[0] + (int64_t)c.oi[1] * p.o_os[1]
               + (int64_t)c.oi[2] * p.o_os[2];
-    c.q_block = p.aux_dim >= 2 ? c.oi[p.aux_dim - 2] : 0;
+    // (no indexing of oi[] with a run-time value: that would push the context into scratch memory)
+    c.q_block = p.aux_dim == 2 ? c.oi[0] : p.aux_dim == 3 ? c.oi[1] : p.aux_dim == 4 ? c.oi[2] : 0;
 }
 
 FFT_DEV uint32_t lds_addr(const fftk_params& p, uint32_t w, uint32_t j)
