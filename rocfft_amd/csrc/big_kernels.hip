@@ -161,7 +161,8 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
 #pragma unroll
         for(int k = 0; k < BIG_EPT; ++k)
         {
-            float2 v = reinterpret_cast<const float2*>(in)[t + 1024 * k];
+            // wave-uniform base per k plus the lane offset t: no per-element address registers
+            float2 v = (reinterpret_cast<const float2*>(in) + 1024 * k)[t];
             r[k]     = inv ? c_swap(v) : v;
         }
     }
@@ -173,12 +174,13 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
         const float2  a  = static_cast<const float2*>(p.half_a)[t];
         const float2* hb = static_cast<const float2*>(p.half_b);
         const float2* hx = reinterpret_cast<const float2*>(in);
+        const uint32_t tr = 1023u - t;
 #pragma unroll
         for(int k = 0; k < BIG_EPT / 2; ++k)
         {
             const uint32_t j  = t + 1024 * k;
-            float2         xa = hx[j];
-            float2         xb = hx[BIG_L - j];
+            float2         xa = (hx + 1024 * k)[t];
+            float2         xb = (hx + (BIG_L - 1024 * k - 1023))[tr];
             float2         zj, zq;
             if(k == 0 && t == 0)
             {
@@ -279,7 +281,7 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
                 v.x *= (float)p.scale;
                 v.y *= (float)p.scale;
             }
-            reinterpret_cast<float2*>(out)[t + 1024 * big_slot_index(s)] = v;
+            (reinterpret_cast<float2*>(out) + 1024 * big_slot_index(s))[t] = v;
         }
         return;
     }
@@ -296,6 +298,7 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
     const float2* hb = static_cast<const float2*>(p.half_b);
     float2*       ho = reinterpret_cast<float2*>(out);
     const float   sc = p.use_scale ? (float)p.scale : 1.0f;
+    const uint32_t tr = 1023u - t;
 #pragma unroll
     for(int s = 0; s < BIG_EPT; ++s)
     {
@@ -340,8 +343,8 @@ __global__ __launch_bounds__(BIG_THREADS) void big32k_kernel(const big_params p)
         o0.y *= sc;
         o1.x *= sc;
         o1.y *= sc;
-        ho[j]         = o0;
-        ho[BIG_L - j] = o1;
+        (ho + 1024 * k)[t]                   = o0;
+        (ho + (BIG_L - 1024 * k - 1023))[tr] = o1;
     }
 }
 
