@@ -10,8 +10,15 @@ namespace
 
 // MODE 0: scalar accesses, every fused operation; 1: vector accesses, every fused operation;
 // 2: the lean path (vector accesses, interleaved complex on both sides)
+// workgroups have up to 256 threads, or 512 when one transform alone needs more than 256
+template <typename Cfg>
+constexpr int fast_block_limit()
+{
+    return Cfg::TPT > 256 ? 512 : 256;
+}
+
 template <typename T, typename Cfg, int MODE>
-__global__ __launch_bounds__(256) void fast_tile_kernel(const fftk_params p)
+__global__ __launch_bounds__(fast_block_limit<Cfg>()) void fast_tile_kernel(const fftk_params p)
 {
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
@@ -69,6 +76,7 @@ const FastEntry g_fast[] = {
     FAST_BOTH(1024, 16, 16, 4, 1)
     FAST_BOTH(2048, 16, 16, 8, 1)
     FAST_BOTH(4096, 16, 16, 16, 1)
+    FAST_BOTH(8192, 16, 16, 8, 4)
 };
 
 const FastEntry* find_fast(int precision, uint32_t n, const uint32_t* radix, uint32_t nf)
@@ -101,7 +109,7 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
                                       size_t lds_bytes, void* stream)
 {
     const FastEntry* e = find_fast(precision, p->n, p->radix, p->nf);
-    if(!e || p->T != e->tpt || p->nthreads > 256 || p->padshift != 4)
+    if(!e || p->T != e->tpt || p->nthreads > (e->tpt > 256 ? 512u : 256u) || p->padshift != 4)
         return (int)hipErrorInvalidValue;
     fast_launch_fn fn = (vec && p->lean) ? e->lean : vec ? e->vec : e->scalar;
     return fn(p, grid, lds_bytes, (hipStream_t)stream);

@@ -599,7 +599,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     {
         k.fast      = 1;
         k.T         = fast_tpt;
-        max_threads = 256;
+        max_threads = fast_tpt > 256 ? 512 : 256;
     }
     size_t   per_tile  = (size_t)k.pitch * esize;
     uint32_t w_threads = floor_pow2(max_threads / k.T);
@@ -827,6 +827,101 @@ static void split_length(uint64_t n, size_t esize, bool column, uint64_t& n1, ui
     n0 = n / best;
 }
 
+static void split_length(uint64_t n, size_t esize, bool column, uint64_t& n1, uint64_t& n0);
+
+static bool factorize(uint64_t n, std::vector<uint32_t>& radix);
+
+static bool fast_kernel_exists(uint64_t n, size_t esize)
+{
+    std::vector<uint32_t> radix;
+    if(!factorize(n, radix) || radix.size() > FFTK_MAX_PASSES)
+        return false;
+    return fftrt_fast_tpt(esize == 16 ? 1 : 0, (uint32_t)n, radix.data(), (uint32_t)radix.size()) != 0;
+}
+
+// Will emit_dim transform a plain complex dimension of length n with one tile pass?
+static bool plain_dim_is_single(uint64_t n, bool column, size_t esize)
+{
+    bool single = column ? column_kernel_length(n, esize) : single_kernel_length(n, esize);
+    // Power-of-two lengths above 4096 have no compile-time-schedule kernel; two passes of those
+    // kernels beat one pass of the run-time-schedule kernel, so split them when that is possible.
+    if(single && g_use_fast && n > 4096 && (n & (n - 1)) == 0 && !fast_kernel_exists(n, esize))
+    {
+        uint64_t a1, a0;
+        split_length(n, esize, column, a1, a0);
+        if(a1 != 0)
+            single = false;
+    }
+    return single;
+}
+
+// n = n1 * n0 for the two-pass scheme: pass A is a strided pass over n1 (it wants a wide
+// tile, so n1 must be a column-kernel length), pass B a row pass over n0 (or another strided
+// pass when the whole dimension is strided).  Prefers factors with compile-time-schedule
+// kernels, then balance.  n1 = 0 when there is no such pair.
+static void split_two(uint64_t n, size_t esize, bool column, uint64_t& n1, uint64_t& n0,
+                      uint64_t max_row = 8192)
+{
+    n1 = n0 = 0;
+    double best_score = -1;
+    for(uint64_t a = 2; a < n; ++a)
+    {
+        if(n % a)
+            continue;
+        uint64_t bq = n / a;
+        if(!column_kernel_length(a, esize))
+            continue;
+        if(!(column ? column_kernel_length(bq, esize) : single_kernel_length(bq, esize)))
+            continue;
+        if(!column && bq > max_row)
+            continue;
+        double score = (fast_kernel_exists(a, esize) ? 2.0 : 0.0) + (fast_kernel_exists(bq, esize) ? 2.0 : 0.0);
+        // balance: prefer a close to sqrt(n) but never a tiny strided factor
+        double ratio = (double)std::min(a, bq) / (double)std::max(a, bq);
+        score += ratio;
+        if(a < 8)
+            score -= 1.0;
+        if(score > best_score)
+        {
+            best_score = score;
+            n1         = a;
+            n0         = bq;
+        }
+    }
+}
+
+// n = n2 * n1 * n0 for the three-pass scheme (n2 and n1 strided passes, n0 as in split_two)
+static void split_three(uint64_t n, size_t esize, bool column, uint64_t& n2, uint64_t& n1,
+                        uint64_t& n0)
+{
+    n2 = n1 = n0 = 0;
+    double best_score = -1;
+    for(uint64_t a = 2; a < n; ++a)
+    {
+        if(n % a || !column_kernel_length(a, esize))
+            continue;
+        uint64_t b1, b0;
+        split_two(n / a, esize, column, b1, b0, 512);
+        if(b1 == 0)
+            split_two(n / a, esize, column, b1, b0);
+        if(b1 == 0)
+            continue;
+        double score = (fast_kernel_exists(a, esize) ? 2.0 : 0.0) + (fast_kernel_exists(b1, esize) ? 2.0 : 0.0)
+                       + (fast_kernel_exists(b0, esize) ? 2.0 : 0.0);
+        // the long factor goes to the row pass; the two strided factors should be similar
+        score += (double)std::min(a, b1) / (double)std::max(a, b1) + (double)b0 / (double)n;
+        if(a < 8)
+            score -= 1.0;
+        if(score > best_score)
+        {
+            best_score = score;
+            n2         = a;
+            n1         = b1;
+            n0         = b0;
+        }
+    }
+}
+
 static bool smooth(uint64_t n)
 {
     std::vector<uint32_t> r;
@@ -895,9 +990,8 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     IoRef blu;
     blu.buf = BUF_BLU;
 
-    bool single = column ? (column_kernel_length(n, esize) || !plain) && single_kernel_length(n, esize)
-                         : single_kernel_length(n, esize);
-    // a strided pass that is not "plain" (fused real/odd handling) stays single if it fits at all
+    // a pass that is not "plain" (fused real/odd handling) stays single if it fits at all
+    bool single = plain ? plain_dim_is_single(n, column, esize) : single_kernel_length(n, esize);
     if(single)
     {
         TileSpec s = base_spec();
@@ -928,12 +1022,76 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     {
         if(!plain)
             fail("this real-transform length needs a decomposition that is not implemented");
-        uint64_t n1, n0;
-        split_length(n, esize, column, n1, n0);
+        // The row pass of the two-pass scheme stores transposed, W rows at a time; beyond 512
+        // points per row W gets too small for coalesced stores, and three passes are faster.
+        uint64_t n1, n0, n2 = 0;
+        split_two(n, esize, column, n1, n0, 512);
         if(n1 == 0)
-            split_length(n, esize, false, n1, n0);
+        {
+            split_three(n, esize, column, n2, n1, n0);
+            if(n2 == 0)
+                split_two(n, esize, column, n1, n0);
+        }
+        if(n2 != 0)
+        {
+            // Three passes, n = n2 * (n1 * n0): a column FFT over the n2 samples that are
+            // R = n1*n0 apart times W_n^{k2 r}; then each contiguous run of R points is
+            // transformed by the two-pass scheme (column FFT over n1 times W_R^{k1 n0'}, row
+            // FFT over n0), the last pass storing result k2 + n2*(k1 + n1*k0).
+            const uint64_t R = n1 * n0;
+            b.need_tmp(lines * n);
+            std::vector<int64_t> pk = packed_strides(n);
+            {
+                TileSpec s = base_spec();
+                s.n        = (uint32_t)n2;
+                s.t_is     = (int64_t)R * t_is;
+                s.t_os     = (int64_t)R * 2;
+                s.src      = src;
+                s.dst      = tmp;
+                s.others.push_back({(uint32_t)R, t_is, 2, true});
+                add_others(s, true, false, pk);
+                s.flags |= FFTK_F_TWIDDLE_STORE;
+                s.ltw       = large_twiddles(n, b.precision, b.dry);
+                s.ltw_shift = large_twiddle_shift(n);
+                s.note      = dims_note("split3 A (column fft over the outer factor + twiddle)", n2);
+                b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+            }
+            {
+                TileSpec s = base_spec();
+                s.n        = (uint32_t)n1;
+                s.t_is = s.t_os = (int64_t)n0 * 2;
+                s.src = s.dst = tmp;
+                s.others.push_back({(uint32_t)n0, 2, 2, true});
+                s.others.push_back({(uint32_t)n2, (int64_t)R * 2, (int64_t)R * 2, false});
+                add_others(s, false, false, pk);
+                s.flags |= FFTK_F_TWIDDLE_STORE;
+                s.ltw       = large_twiddles(R, b.precision, b.dry);
+                s.ltw_shift = large_twiddle_shift(R);
+                s.note      = dims_note("split3 B (column fft over the middle factor + twiddle)", n1);
+                b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+            }
+            {
+                TileSpec s = base_spec();
+                s.n        = (uint32_t)n0;
+                s.t_is     = 2;
+                s.t_os     = (int64_t)(n1 * n2) * t_os;
+                s.src      = tmp;
+                s.dst      = dst;
+                s.others.push_back({(uint32_t)n1, (int64_t)n0 * 2, (int64_t)n2 * t_os, false});
+                s.others.push_back({(uint32_t)n2, (int64_t)R * 2, t_os, false});
+                add_others(s, false, true, pk);
+                if(ops.has_scale)
+                {
+                    s.flags |= FFTK_F_SCALE;
+                    s.scale = ops.scale;
+                }
+                s.note = dims_note("split3 C (row fft, doubly transposed store)", n0);
+                b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+            }
+            return;
+        }
         if(n1 == 0)
-            fail("length too large for a two-pass decomposition");
+            fail("length too large for the two- and three-pass decompositions");
         // pass A: for every n0' an n1-point FFT over the stride-n0 samples, times W_n^{k1 n0'},
         // written to scratch at [line][k1*n0 + n0']
         // pass B: for every k1 an n0-point FFT over n0', written to dst at k0*n1 + k1
@@ -1375,7 +1533,7 @@ static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t 
     for(size_t i = 0; i < rank; ++i)
         if(i != d && len[i] > 1 && (src.stride[i] < src.stride[d]))
             d_column = true;
-    if(!(d_column ? column_kernel_length(len[d], esize) : single_kernel_length(len[d], esize)))
+    if(!plain_dim_is_single(len[d], d_column, esize))
         return false;
     if(src.io.planar || out.io.planar)
         return false;

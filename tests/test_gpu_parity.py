@@ -70,13 +70,20 @@ def test_long_1d(gpu, n):
 
 
 @pytest.mark.parametrize("lengths", [[8, 8], [64, 64], [100, 30], [17, 19], [1024, 1024], [4096, 64], [64, 4096],
-                                     [8, 8, 8], [16, 8, 4], [30, 20, 10], [128, 32, 8], [5, 7, 9], [64, 64, 64],
+                                     [8, 8, 8], [16, 8, 4], [30, 20, 10], [128, 32, 8], [5, 7, 9], [8192, 4], [4, 8192], [64, 64, 64],
                                      [128, 128, 128], [512, 16, 16], [16, 512, 4], [8, 4, 512], [1, 8], [8, 1, 4]])
 def test_multi_dim(gpu, lengths):
     lib, be = gpu
     for kind in range(4):
         H.check(lib, be, kind, lengths, 2, B.DOUBLE)
         H.check(lib, be, kind, lengths, 1, B.SINGLE, inplace=True)
+
+
+def test_large_square_2d(gpu):
+    # both dimensions beyond the longest single-kernel length
+    lib, be = gpu
+    H.check(lib, be, B.COMPLEX_FORWARD, [8192, 8192], 1, B.SINGLE)
+    H.check(lib, be, B.COMPLEX_INVERSE, [4096, 2048], 2, B.DOUBLE, inplace=True)
 
 
 def test_layouts(gpu):

@@ -261,7 +261,7 @@ def test_long_1d(emu, lengths):
 
 @pytest.mark.parametrize("lengths", [[8, 8], [64, 64], [100, 30], [30, 100], [17, 19], [1024, 1024], [4, 2048],
                                      [2048, 4], [8, 8, 8], [16, 8, 4], [4, 8, 16], [30, 20, 10], [128, 32, 8],
-                                     [5, 7, 9], [64, 64, 64], [2, 2, 2], [1, 8], [8, 1, 4]])
+                                     [5, 7, 9], [8192, 4], [4, 8192], [64, 64, 64], [2, 2, 2], [1, 8], [8, 1, 4]])
 def test_multi_dim(emu, lengths):
     for kind in range(4):
         H.check(emu, HOST, kind, lengths, 2, B.DOUBLE)
