@@ -372,4 +372,131 @@ struct Butterfly<T, 16>
     }
 };
 
+// Composite radix R = A*B from two smaller butterflies (Cooley-Tukey with n = B a + b,
+// k = k1 + A k2):
+//   y[b][k1]      = sum_a x[B a + b] W_A^{a k1}
+//   X[k1 + A k2]  = sum_b W_B^{b k2} (W_R^{b k1} y[b][k1])
+// cs[m], sn[m] = cos, sin(2 pi m / R); the table indices are compile-time after unrolling.
+template <typename T, int A, int B>
+struct CompositeButterfly
+{
+    typedef typename cplx_of<T>::type C;
+    static FFT_DEV void               run(C* r, const T* cs, const T* sn)
+    {
+        constexpr int R = A * B;
+        C             y[B][A];
+#pragma unroll
+        for(int b = 0; b < B; ++b)
+        {
+#pragma unroll
+            for(int a = 0; a < A; ++a)
+                y[b][a] = r[B * a + b];
+            Butterfly<T, A>::run(y[b]);
+        }
+#pragma unroll
+        for(int b = 1; b < B; ++b)
+#pragma unroll
+            for(int k1 = 1; k1 < A; ++k1)
+            {
+                const int m = (b * k1) % R;
+                C         w;
+                w.x      = cs[m];
+                w.y      = -sn[m];
+                y[b][k1] = c_mul(y[b][k1], w);
+            }
+#pragma unroll
+        for(int k1 = 0; k1 < A; ++k1)
+        {
+            C z[B];
+#pragma unroll
+            for(int b = 0; b < B; ++b)
+                z[b] = y[b][k1];
+            Butterfly<T, B>::run(z);
+#pragma unroll
+            for(int k2 = 0; k2 < B; ++k2)
+                r[k1 + A * k2] = z[k2];
+        }
+    }
+};
+
+template <typename T>
+struct Butterfly<T, 6>
+{
+    typedef typename cplx_of<T>::type C;
+    static FFT_DEV void               run(C* r)
+    {
+        const T cs[6] = {(T)1.0,
+                         (T)0.5,
+                         (T)-0.5,
+                         (T)-1.0,
+                         (T)-0.5,
+                         (T)0.5};
+        const T sn[6] = {(T)0.0,
+                         (T)0.866025403784438646763723170752936183,
+                         (T)0.866025403784438646763723170752936183,
+                         (T)4.13406421965279764729938061032096894e-43,
+                         (T)-0.866025403784438646763723170752936183,
+                         (T)-0.866025403784438646763723170752936183};
+        CompositeButterfly<T, 3, 2>::run(r, cs, sn);
+    }
+};
+
+template <typename T>
+struct Butterfly<T, 9>
+{
+    typedef typename cplx_of<T>::type C;
+    static FFT_DEV void               run(C* r)
+    {
+        const T cs[9] = {(T)1.0,
+                         (T)0.766044443118978035202392650555416674,
+                         (T)0.173648177666930348851716626769314796,
+                         (T)-0.5,
+                         (T)-0.93969262078590838405410927732473147,
+                         (T)-0.93969262078590838405410927732473147,
+                         (T)-0.5,
+                         (T)0.173648177666930348851716626769314796,
+                         (T)0.766044443118978035202392650555416674};
+        const T sn[9] = {(T)0.0,
+                         (T)0.642787609686539326322643409907263433,
+                         (T)0.984807753012208059366743024589523014,
+                         (T)0.866025403784438646763723170752936183,
+                         (T)0.342020143325668733044099614682259581,
+                         (T)-0.342020143325668733044099614682259581,
+                         (T)-0.866025403784438646763723170752936183,
+                         (T)-0.984807753012208059366743024589523014,
+                         (T)-0.642787609686539326322643409907263433};
+        CompositeButterfly<T, 3, 3>::run(r, cs, sn);
+    }
+};
+
+template <typename T>
+struct Butterfly<T, 10>
+{
+    typedef typename cplx_of<T>::type C;
+    static FFT_DEV void               run(C* r)
+    {
+        const T cs[10] = {(T)1.0,
+                          (T)0.809016994374947424102293417182819059,
+                          (T)0.309016994374947424102293417182819059,
+                          (T)-0.309016994374947424102293417182819059,
+                          (T)-0.809016994374947424102293417182819059,
+                          (T)-1.0,
+                          (T)-0.809016994374947424102293417182819059,
+                          (T)-0.309016994374947424102293417182819059,
+                          (T)0.309016994374947424102293417182819059,
+                          (T)0.809016994374947424102293417182819059};
+        const T sn[10] = {(T)0.0,
+                          (T)0.587785252292473129168705954639072769,
+                          (T)0.951056516295153572116439333379382143,
+                          (T)0.951056516295153572116439333379382143,
+                          (T)0.587785252292473129168705954639072769,
+                          (T)4.13406421965279764729938061032096894e-43,
+                          (T)-0.587785252292473129168705954639072769,
+                          (T)-0.951056516295153572116439333379382143,
+                          (T)-0.951056516295153572116439333379382143,
+                          (T)-0.587785252292473129168705954639072769};
+        CompositeButterfly<T, 5, 2>::run(r, cs, sn);
+    }
+};
+
 #endif

@@ -2,7 +2,7 @@
 //
 // Same tile model as tile_core.h (a workgroup owns W transforms of length N),
 // but length, radices and threads per transform are template parameters, every
-// thread keeps its EPT = max radix elements in registers for the whole kernel,
+// thread keeps its (at most FFTK_REG_ELEMS) elements in registers for the whole kernel,
 // and -- where the lane order matches the fast axis in memory -- the first pass
 // loads straight from global memory into registers and the last pass stores
 // straight from registers, so LDS is only used for the exchanges between passes.
@@ -18,7 +18,10 @@
 
 #include "tile_core.h"
 
-template <int N_, int R0_, int R1_, int R2_, int R3_>
+// TPT_ = 0 takes the fewest threads per transform that the register budget allows; a larger
+// value spreads a transform over more lanes (longer contiguous runs per access, fewer
+// registers per thread).
+template <int N_, int R0_, int R1_, int R2_, int R3_, int TPT_ = 0>
 struct FastCfg
 {
     static constexpr int N  = N_;
@@ -28,13 +31,34 @@ struct FastCfg
     {
         return a > b ? a : b;
     }
-    static constexpr int RMAX = max2(max2(R0_, R1_), max2(R2_, R3_));
-    static constexpr int TPT  = N_ / RMAX; // threads per transform
-    static constexpr int EPT  = RMAX;      // elements per thread
     static constexpr int radix(int p)
     {
         return p == 0 ? R0_ : p == 1 ? R1_ : p == 2 ? R2_ : R3_;
     }
+    // threads one pass of radix r needs when a thread holds at most FFTK_REG_ELEMS values:
+    // the same rule the planner applies to the generic kernel
+    static constexpr int need(int r)
+    {
+        return r > 1 ? (N_ / r + FFTK_REG_ELEMS / r - 1) / (FFTK_REG_ELEMS / r) : 1;
+    }
+    static constexpr int TPT_MIN = max2(max2(need(R0_), need(R1_)), max2(need(R2_), need(R3_)));
+    static constexpr int TPT     = TPT_ ? TPT_ : TPT_MIN; // threads per transform
+    static_assert(TPT >= TPT_MIN, "too few threads per transform for the register budget");
+    // butterflies a thread computes in pass p; when N/radix is no multiple of TPT the
+    // last slot of the higher lanes is idle (live() tells)
+    static constexpr int S(int p)
+    {
+        return (N_ / radix(p) + TPT - 1) / TPT;
+    }
+    static constexpr bool exact(int p)
+    {
+        return (N_ / radix(p)) % TPT == 0;
+    }
+    static constexpr int elems(int p)
+    {
+        return p < NP ? S(p) * radix(p) : 0;
+    }
+    static constexpr int EPT = max2(max2(elems(0), elems(1)), max2(elems(2), elems(3))); // register elements per thread
     static constexpr int cum(int p)
     {
         return p == 0 ? 1 : p == 1 ? R0_ : p == 2 ? R0_ * R1_ : R0_ * R1_ * R2_;
@@ -47,14 +71,20 @@ struct FastCfg
     static constexpr int PADSHIFT = 4;
     static constexpr int PITCH    = (N_ + ((N_ - 1) >> PADSHIFT) + 1) | 1;
     static_assert(N_ == R0_ * R1_ * R2_ * R3_, "radices must multiply to N");
-    static_assert(RMAX % R0_ == 0 && RMAX % R1_ == 0 && RMAX % R2_ == 0 && RMAX % R3_ == 0,
-                  "every radix must divide the largest one");
+    static_assert(EPT <= FFTK_REG_ELEMS, "a thread holds at most FFTK_REG_ELEMS values");
 };
 
 template <typename Cfg>
 FFT_DEV uint32_t fk_addr(uint32_t w, uint32_t j)
 {
     return w * Cfg::PITCH + j + (j >> Cfg::PADSHIFT);
+}
+
+// does lane tt have a butterfly in slot s of pass P?
+template <typename Cfg, int P>
+FFT_DEV bool fk_live(uint32_t tt, int s)
+{
+    return Cfg::exact(P) || tt + (uint32_t)(s * Cfg::TPT) < (uint32_t)(Cfg::N / Cfg::radix(P));
 }
 
 // position of element (butterfly slot s, input k) of pass P held by lane tt
@@ -79,12 +109,15 @@ FFT_DEV void fk_read(const typename cplx_of<T>::type* lds, uint32_t w, uint32_t 
                      typename cplx_of<T>::type* r)
 {
     constexpr int R = Cfg::radix(P);
-    constexpr int S = Cfg::EPT / R;
+    constexpr int S = Cfg::S(P);
 #pragma unroll
     for(int s = 0; s < S; ++s)
+        if(fk_live<Cfg, P>(tt, s))
+        {
 #pragma unroll
-        for(int k = 0; k < R; ++k)
-            r[s * R + k] = lds[fk_addr<Cfg>(w, fk_in_pos<Cfg, P>(tt, s, k))];
+            for(int k = 0; k < R; ++k)
+                r[s * R + k] = lds[fk_addr<Cfg>(w, fk_in_pos<Cfg, P>(tt, s, k))];
+        }
 }
 
 template <typename T, typename Cfg, int P>
@@ -92,12 +125,15 @@ FFT_DEV void fk_write(typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
                       const typename cplx_of<T>::type* r)
 {
     constexpr int R = Cfg::radix(P);
-    constexpr int S = Cfg::EPT / R;
+    constexpr int S = Cfg::S(P);
 #pragma unroll
     for(int s = 0; s < S; ++s)
+        if(fk_live<Cfg, P>(tt, s))
+        {
 #pragma unroll
-        for(int k = 0; k < R; ++k)
-            lds[fk_addr<Cfg>(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
+            for(int k = 0; k < R; ++k)
+                lds[fk_addr<Cfg>(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
+        }
 }
 
 template <typename T, typename Cfg, int P>
@@ -105,11 +141,13 @@ FFT_DEV void fk_compute(const fftk_params& p, uint32_t tt, typename cplx_of<T>::
 {
     typedef typename cplx_of<T>::type C;
     constexpr int                     R = Cfg::radix(P);
-    constexpr int                     S = Cfg::EPT / R;
+    constexpr int                     S = Cfg::S(P);
     constexpr uint32_t                c = Cfg::cum(P);
 #pragma unroll
     for(int s = 0; s < S; ++s)
     {
+        if(!fk_live<Cfg, P>(tt, s))
+            continue;
         if(P > 0)
         {
             const C* tw = static_cast<const C*>(p.tw) + Cfg::twoff(P);
@@ -186,11 +224,14 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     constexpr int                     N    = Cfg::N;
     constexpr int                     LAST = Cfg::NP - 1;
     constexpr int                     RL   = Cfg::radix(LAST);
-    constexpr int                     SL   = Cfg::EPT / RL;
+    constexpr int                     SL   = Cfg::S(LAST);
     constexpr int                     CL   = N / RL; // output (s,k) of the last pass is element tt + s*TPT + k*CL
     constexpr int                     R0   = Cfg::radix(0);
-    constexpr int                     S0   = Cfg::EPT / R0;
+    constexpr int                     S0   = Cfg::S(0);
     constexpr int                     M0   = N / R0; // input (s,k) of pass 0 is element tt + s*TPT + k*M0
+    constexpr int                     PAIRS      = (N + 1) / 2; // bins j paired with N-j (j = 0 pairs with N)
+    constexpr int                     PAIR_IT    = (PAIRS + Cfg::TPT - 1) / Cfg::TPT;
+    constexpr bool                    PAIR_EXACT = PAIRS % Cfg::TPT == 0;
     const bool                        ok   = active && (c.tile0 + w < p.tile_cnt);
     const bool                        inv  = p.dir > 0;
     const C*       src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
@@ -203,17 +244,20 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     if(p.load_op == FFTK_LOAD_C2R_PRE)
     {
         // Hermitian bins -> half-length complex input (library/src/device/kernels/
-        // real2complex_device.h:212-254).  A thread takes the pairs (j, N-j), j = tt + TPT*i < N/2,
-        // writes z_j and z_{N-j} to LDS in natural order; pass 0 then reads from LDS.
+        // real2complex_device.h:212-254).  A thread takes the pairs (j, N-j), j = tt + TPT*i < (N+1)/2,
+        // writes z_j and z_{N-j} to LDS in natural order; pass 0 then reads from LDS.  An even N
+        // has the unpaired bin N/2 besides.
         const C*       htw = static_cast<const C*>(p.half_tw);
         const uint32_t wo  = w * p.w_is_c;
         if(ok)
         {
 #pragma unroll
-            for(int i = 0; i < Cfg::EPT / 2; ++i)
+            for(int i = 0; i < PAIR_IT; ++i)
             {
                 const uint32_t j  = tt + i * Cfg::TPT;
                 const uint32_t jq = N - j;
+                if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
+                    continue;
                 C              a  = src[j * p.t_is_c + wo];
                 C              bq = src[jq * p.t_is_c + wo];
                 C              zj, zq;
@@ -235,7 +279,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 }
                 lds[fk_addr<Cfg>(w, j)] = c_swap(zj);
             }
-            if(tt == 0)
+            if(N % 2 == 0 && tt == 0)
             {
                 C a = src[(N / 2) * p.t_is_c + wo];
                 C z;
@@ -268,7 +312,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     {
                         const uint32_t j     = tt + s * Cfg::TPT + k * M0;
                         const uint32_t idx   = j * p.chirp_js + q * p.chirp_qs;
-                        const bool     valid = idx < p.blu_n;
+                        const bool     valid = idx < p.blu_n && fk_live<Cfg, 0>(tt, s);
                         const uint32_t off   = valid ? j * p.t_is_c + w * p.w_is_c : 0u;
                         r[s * R0 + k]        = src[off];
                         ch[s * R0 + k]       = chirp[valid ? idx : 0u];
@@ -298,7 +342,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     for(int k = 0; k < R0; ++k)
                     {
                         const C* pk = src + (uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c;
-                        r[s * R0 + k] = pk[li];
+                        if(fk_live<Cfg, 0>(tt, s))
+                            r[s * R0 + k] = pk[li];
                     }
             }
             if(inv)
@@ -328,7 +373,9 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 for(int k = 0; k < RL; ++k)
                 {
                     const uint32_t j = tt + s * Cfg::TPT + k * CL;
-                    C              v = r[s * RL + k];
+                    if(!fk_live<Cfg, LAST>(tt, s))
+                        continue;
+                    C v = r[s * RL + k];
                     if(ok)
                         v = c_mul(v, cb[j]);
                     lds[fk_addr<Cfg>(w, j)] = c_swap(v);
@@ -358,10 +405,12 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             const uint32_t wo  = w * p.w_os_c;
             const T        sc  = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
 #pragma unroll
-            for(int i = 0; i < Cfg::EPT / 2; ++i)
+            for(int i = 0; i < PAIR_IT; ++i)
             {
                 const uint32_t j  = tt + i * Cfg::TPT;
                 const uint32_t jq = N - j;
+                if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
+                    continue;
                 C              zp = lds[fk_addr<Cfg>(w, j)];
                 C              o0, o1;
                 if(j == 0)
@@ -392,7 +441,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 dst[j * p.t_os_c + wo]  = o0;
                 dst[jq * p.t_os_c + wo] = o1;
             }
-            if(tt == 0)
+            if(N % 2 == 0 && tt == 0)
             {
                 C z = lds[fk_addr<Cfg>(w, N / 2)];
                 C o;
@@ -433,7 +482,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             for(int s = 0; s < SL; ++s)
 #pragma unroll
                 for(int k = 0; k < RL; ++k)
-                    r[s * RL + k] = lds[fk_addr<Cfg>(ow, ot + s * Cfg::TPT + k * CL)];
+                    if(fk_live<Cfg, LAST>(ot, s))
+                        r[s * RL + k] = lds[fk_addr<Cfg>(ow, ot + s * Cfg::TPT + k * CL)];
         }
     }
     const uint32_t oq = p.aux_dim == 1 ? c.tile0 + ow : c.q_block;
@@ -478,7 +528,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 {
                     const uint32_t j   = ot + s * Cfg::TPT + k * CL;
                     const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
-                    ch[s * RL + k]     = chirp[idx < p.blu_n ? idx : 0u];
+                    ch[s * RL + k]     = chirp[(idx < p.blu_n && fk_live<Cfg, LAST>(ot, s)) ? idx : 0u];
                 }
 #pragma unroll
             for(int s = 0; s < SL; ++s)
@@ -488,7 +538,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     const uint32_t j   = ot + s * Cfg::TPT + k * CL;
                     const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
                     C v = cj ? c_mul(r[s * RL + k], ch[s * RL + k]) : c_mulc(r[s * RL + k], ch[s * RL + k]);
-                    if(idx < p.blu_n && j < p.n_out)
+                    if(idx < p.blu_n && j < p.n_out && fk_live<Cfg, LAST>(ot, s))
                     {
                         C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
                         pk[lo] = v;
@@ -502,8 +552,9 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
 #pragma unroll
                 for(int k = 0; k < RL; ++k)
                 {
-                    C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
-                    pk[lo] = r[s * RL + k];
+                    C* pk = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
+                    if(fk_live<Cfg, LAST>(ot, s))
+                        pk[lo] = r[s * RL + k];
                 }
         }
     }
@@ -515,9 +566,9 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
     typedef typename cplx_of<T>::type C;
     constexpr int                     LAST = Cfg::NP - 1;
     constexpr int                     RL   = Cfg::radix(LAST);
-    constexpr int                     SL   = Cfg::EPT / RL;
+    constexpr int                     SL   = Cfg::S(LAST);
     constexpr int                     R0   = Cfg::radix(0);
-    constexpr int                     S0   = Cfg::EPT / R0;
+    constexpr int                     S0   = Cfg::S(0);
     const uint32_t                    tid  = threadIdx.x;
     TileCtx<T>                        c;
     tile_decode<T>(p, blockIdx.x, c);
@@ -548,7 +599,8 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
             for(int s = 0; s < S0; ++s)
 #pragma unroll
                 for(int k = 0; k < R0; ++k)
-                    r[s * R0 + k] = fetch_elem<T, VEC>(p, c, w, fk_in_pos<Cfg, 0>(tt, s, k));
+                    if(fk_live<Cfg, 0>(tt, s))
+                        r[s * R0 + k] = fetch_elem<T, VEC>(p, c, w, fk_in_pos<Cfg, 0>(tt, s, k));
         }
         lds_busy = false;
     }
@@ -577,7 +629,9 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
                 for(int k = 0; k < RL; ++k)
                 {
                     uint32_t j = fk_out_pos<Cfg, LAST>(tt, s, k);
-                    C        v = r[s * RL + k];
+                    if(!fk_live<Cfg, LAST>(tt, s))
+                        continue;
+                    C v = r[s * RL + k];
                     if(valid)
                         v = c_mul(v, static_cast<const C*>(p.convb)[j + q * p.convb_qs]);
                     lds[fk_addr<Cfg>(w, j)] = c_swap(v);
@@ -596,7 +650,8 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
             for(int s = 0; s < SL; ++s)
 #pragma unroll
                 for(int k = 0; k < RL; ++k)
-                    emit_elem<T, VEC>(p, c, w, fk_out_pos<Cfg, LAST>(tt, s, k), r[s * RL + k]);
+                    if(fk_live<Cfg, LAST>(tt, s))
+                        emit_elem<T, VEC>(p, c, w, fk_out_pos<Cfg, LAST>(tt, s, k), r[s * RL + k]);
         }
     }
     else

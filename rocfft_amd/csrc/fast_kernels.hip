@@ -1,9 +1,21 @@
 // fast_kernels.hip -- instantiations of the compile-time-schedule tile kernel
-// (fast_core.h) for the power-of-two lengths, and their registry.
+// (fast_core.h) for the lengths listed in fast_schedules.h, and their registry.
+//
+// The file is compiled FAST_SLICES times with -DFAST_SLICE=0..FAST_SLICES-1; every
+// translation unit instantiates the kernels of its slice of the list, and slice 0 also
+// holds the lookup over all slices.
 #include "fast_core.h"
+#include "fast_registry.h"
 #include "gpu_rt.h"
 #include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cstdlib>
 #include <mutex>
+#include <vector>
+
+#ifndef FAST_SLICE
+#error "compile with -DFAST_SLICE=<n>"
+#endif
 
 namespace
 {
@@ -25,10 +37,8 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>()) void fast_tile_kernel(cons
     fast_tile_body<T, Cfg, MODE != 0, MODE == 2>(p, reinterpret_cast<C*>(smem_raw));
 }
 
-typedef int (*fast_launch_fn)(const fftk_params*, uint32_t, size_t, hipStream_t);
-
 template <typename T, typename Cfg, int MODE>
-int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, hipStream_t stream)
+int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* stream)
 {
     auto kernel = fast_tile_kernel<T, Cfg, MODE>;
     if(lds_bytes > 64 * 1024)
@@ -44,73 +54,166 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, hipStream
         if(rc)
             return rc;
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p->nthreads), lds_bytes, stream, *p);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(p->nthreads), lds_bytes, (hipStream_t)stream, *p);
     return (int)hipGetLastError();
 }
 
-struct FastEntry
-{
-    int            precision;
-    uint32_t       n;
-    uint32_t       radix[4];
-    uint32_t       tpt;
-    fast_launch_fn lean, vec, scalar;
+// all_modes = 1: the three variants; 0: the lean one only
+#define FAST_ONE_1(T, P, N, A, B, C, D, TT)                                                            \
+    {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 0>},
+#define FAST_ONE_0(T, P, N, A, B, C, D, TT)                                                            \
+    {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
+     nullptr, nullptr},
+#define FAST_ENTRY(FULL, N, A, B, C, D, TTF, TTD) \
+    FAST_ONE_##FULL(float, 0, N, A, B, C, D, TTF) FAST_ONE_##FULL(double, 1, N, A, B, C, D, TTD)
+
+#define FAST_PICK_0(...)
+#define FAST_PICK_1(...)
+#define FAST_PICK_2(...)
+#define FAST_PICK_3(...)
+#define FAST_PICK_4(...)
+#define FAST_PICK_5(...)
+#define FAST_PICK_6(...)
+#define FAST_PICK_7(...)
+#if FAST_SLICE == 0
+#undef FAST_PICK_0
+#define FAST_PICK_0(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 1
+#undef FAST_PICK_1
+#define FAST_PICK_1(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 2
+#undef FAST_PICK_2
+#define FAST_PICK_2(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 3
+#undef FAST_PICK_3
+#define FAST_PICK_3(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 4
+#undef FAST_PICK_4
+#define FAST_PICK_4(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 5
+#undef FAST_PICK_5
+#define FAST_PICK_5(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 6
+#undef FAST_PICK_6
+#define FAST_PICK_6(...) FAST_ENTRY(__VA_ARGS__)
+#elif FAST_SLICE == 7
+#undef FAST_PICK_7
+#define FAST_PICK_7(...) FAST_ENTRY(__VA_ARGS__)
+#else
+#error "FAST_SLICE out of range"
+#endif
+#define FAST_SCHED(SLICE, ...) FAST_PICK_##SLICE(__VA_ARGS__)
+
+const FastEntry g_slice[] = {
+#include "fast_schedules.h"
 };
+static_assert(FAST_SLICES == 8, "the FAST_PICK_ list above covers eight slices");
 
-#define FAST_ONE(T, P, N, A, B, C, D)                                                              \
-    {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D>, 2>,  \
-     &launch_fast<T, FastCfg<N, A, B, C, D>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D>, 0>},
-#define FAST_BOTH(N, A, B, C, D) FAST_ONE(float, 0, N, A, B, C, D) FAST_ONE(double, 1, N, A, B, C, D)
+} // namespace
 
-// the schedules the planner's factorisation produces for powers of two
-const FastEntry g_fast[] = {
-    FAST_BOTH(2, 2, 1, 1, 1)
-    FAST_BOTH(4, 4, 1, 1, 1)
-    FAST_BOTH(8, 8, 1, 1, 1)
-    FAST_BOTH(16, 16, 1, 1, 1)
-    FAST_BOTH(32, 8, 4, 1, 1)
-    FAST_BOTH(64, 16, 4, 1, 1)
-    FAST_BOTH(128, 16, 8, 1, 1)
-    FAST_BOTH(256, 16, 16, 1, 1)
-    FAST_BOTH(512, 16, 8, 4, 1)
-    FAST_BOTH(1024, 16, 16, 4, 1)
-    FAST_BOTH(2048, 16, 16, 8, 1)
-    FAST_BOTH(4096, 16, 16, 16, 1)
-    FAST_BOTH(8192, 16, 16, 8, 4)
-};
+#define FAST_SLICE_FN2(I) fftrt_fast_slice_##I
+#define FAST_SLICE_FN(I) FAST_SLICE_FN2(I)
 
-const FastEntry* find_fast(int precision, uint32_t n, const uint32_t* radix, uint32_t nf)
+extern "C" const FastEntry* FAST_SLICE_FN(FAST_SLICE)(int* count)
 {
-    if(nf < 1 || nf > 4)
+    *count = (int)(sizeof(g_slice) / sizeof(g_slice[0]));
+    return g_slice;
+}
+
+#if FAST_SLICE == 0
+extern "C" const FastEntry* fftrt_fast_slice_1(int*);
+extern "C" const FastEntry* fftrt_fast_slice_2(int*);
+extern "C" const FastEntry* fftrt_fast_slice_3(int*);
+extern "C" const FastEntry* fftrt_fast_slice_4(int*);
+extern "C" const FastEntry* fftrt_fast_slice_5(int*);
+extern "C" const FastEntry* fftrt_fast_slice_6(int*);
+extern "C" const FastEntry* fftrt_fast_slice_7(int*);
+
+namespace
+{
+
+// All entries, sorted by (precision, n).  The list normally holds one schedule per length;
+// a tuning build may hold several, and ROCFFT_AMD_FAST_VARIANT=<v> then selects the
+// (v mod count)-th of each length.
+const std::vector<const FastEntry*>& fast_index()
+{
+    static std::vector<const FastEntry*> index;
+    static std::once_flag                once;
+    std::call_once(once, []() {
+        typedef const FastEntry* (*slice_fn)(int*);
+        const slice_fn slices[FAST_SLICES]
+            = {fftrt_fast_slice_0, fftrt_fast_slice_1, fftrt_fast_slice_2, fftrt_fast_slice_3,
+               fftrt_fast_slice_4, fftrt_fast_slice_5, fftrt_fast_slice_6, fftrt_fast_slice_7};
+        for(slice_fn f : slices)
+        {
+            int              cnt = 0;
+            const FastEntry* e   = f(&cnt);
+            for(int i = 0; i < cnt; ++i)
+                index.push_back(e + i);
+        }
+        std::stable_sort(index.begin(), index.end(), [](const FastEntry* a, const FastEntry* b) {
+            return a->precision != b->precision ? a->precision < b->precision : a->n < b->n;
+        });
+        const char*  env     = getenv("ROCFFT_AMD_FAST_VARIANT");
+        const size_t variant = env ? (size_t)strtoul(env, nullptr, 10) : 0;
+        std::vector<const FastEntry*> picked;
+        for(size_t i = 0; i < index.size();)
+        {
+            size_t j = i;
+            while(j < index.size() && index[j]->precision == index[i]->precision && index[j]->n == index[i]->n)
+                ++j;
+            picked.push_back(index[i + variant % (j - i)]);
+            i = j;
+        }
+        index.swap(picked);
+    });
+    return index;
+}
+
+const FastEntry* find_fast(int precision, uint32_t n)
+{
+    const auto& index = fast_index();
+    auto        it    = std::lower_bound(index.begin(), index.end(), n, [&](const FastEntry* e, uint32_t v) {
+        return e->precision != precision ? e->precision < precision : e->n < v;
+    });
+    if(it == index.end() || (*it)->precision != precision || (*it)->n != n)
         return nullptr;
-    for(const FastEntry& e : g_fast)
-    {
-        if(e.precision != precision || e.n != n)
-            continue;
-        bool same = true;
-        for(uint32_t i = 0; i < 4; ++i)
-            same = same && e.radix[i] == (i < nf ? radix[i] : 1u);
-        if(same)
-            return &e;
-    }
-    return nullptr;
+    return *it;
 }
 
 } // namespace
 
-extern "C" uint32_t fftrt_fast_tpt(int precision, uint32_t n, const uint32_t* radix, uint32_t nf)
+extern "C" uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* radix, uint32_t* nf)
 {
-    const FastEntry* e = find_fast(precision, n, radix, nf);
-    return e ? e->tpt : 0;
+    const FastEntry* e = find_fast(precision, n);
+    if(!e)
+        return 0;
+    uint32_t cnt = 0;
+    for(uint32_t i = 0; i < 4; ++i)
+        if(e->radix[i] > 1)
+            radix[cnt++] = e->radix[i];
+    *nf = cnt;
+    return e->tpt;
 }
 
-// called by fftrt_launch_tile (kernels.hip) when the plan asked for the fast kernel
+// called by fftrt_launch_tile (kernels.hip) when the plan asked for the fast kernel;
+// returns FFTRT_NO_FAST_VARIANT when this access mode has no compiled variant
 extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
                                       size_t lds_bytes, void* stream)
 {
-    const FastEntry* e = find_fast(precision, p->n, p->radix, p->nf);
+    const FastEntry* e = find_fast(precision, p->n);
     if(!e || p->T != e->tpt || p->nthreads > (e->tpt > 256 ? 512u : 256u) || p->padshift != 4)
         return (int)hipErrorInvalidValue;
+    uint32_t cnt = 0;
+    for(uint32_t i = 0; i < 4; ++i)
+        if(e->radix[i] > 1 && (cnt >= p->nf || p->radix[cnt++] != e->radix[i]))
+            return (int)hipErrorInvalidValue;
+    if(cnt != p->nf)
+        return (int)hipErrorInvalidValue;
     fast_launch_fn fn = (vec && p->lean) ? e->lean : vec ? e->vec : e->scalar;
-    return fn(p, grid, lds_bytes, (hipStream_t)stream);
+    if(!fn)
+        return FFTRT_NO_FAST_VARIANT;
+    return fn(p, grid, lds_bytes, stream);
 }
+#endif

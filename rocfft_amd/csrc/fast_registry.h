@@ -1,0 +1,24 @@
+// fast_registry.h -- table entry of a compile-time-schedule tile kernel.  Each slice of
+// fast_kernels.hip exports its entries; the lookup (fast_kernels.hip, slice 0) merges them.
+#ifndef ROCFFT_AMD_FAST_REGISTRY_H
+#define ROCFFT_AMD_FAST_REGISTRY_H
+
+#include "kparams.h"
+#include <stddef.h>
+#include <stdint.h>
+
+typedef int (*fast_launch_fn)(const struct fftk_params*, uint32_t grid, size_t lds_bytes, void* stream);
+
+struct FastEntry
+{
+    int      precision; // 0 single, 1 double
+    uint32_t n;
+    uint32_t radix[4]; // unused passes are 1
+    uint32_t tpt; // threads per transform
+    // lean: vector accesses, interleaved complex on both sides; vec: vector accesses, every
+    // fused operation; scalar: scalar accesses.  A missing variant is null and the generic
+    // kernel runs instead.
+    fast_launch_fn lean, vec, scalar;
+};
+
+#endif

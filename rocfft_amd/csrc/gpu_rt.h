@@ -27,9 +27,14 @@ int fftrt_device_sync(void);
 // 1 when `stream` is being captured into a graph
 int fftrt_stream_capturing(void* stream);
 
-// Threads per transform of the compiled-in fast kernel for this exact pass
-// schedule, or 0 when there is none (the generic kernel is used then).
-uint32_t fftrt_fast_tpt(int precision, uint32_t n, const uint32_t* radix, uint32_t nf);
+// Pass schedule of the compile-time-schedule ("fast") kernel for length n: writes its
+// radices (at most 4) and their count and returns its threads per transform, or returns 0
+// when there is no such kernel (the generic kernel runs the planner's own factorisation
+// then).  The threads per transform follow the generic kernel's rule, so a pass planned
+// for a fast kernel can run on the generic one when an access mode has no fast variant.
+uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* radix, uint32_t* nf);
+// returned by the fast launcher when the requested access mode has no compiled variant
+#define FFTRT_NO_FAST_VARIANT (-2)
 
 // precision: 0 = float, 1 = double.  vec: 1 when both sides are interleaved
 // complex and can move (re, im) pairs with one access.

@@ -31,8 +31,11 @@ __device__ __forceinline__ void run_passes(const fftk_params&         p,
             FFTK_CASE(3)
             FFTK_CASE(4)
             FFTK_CASE(5)
+            FFTK_CASE(6)
             FFTK_CASE(7)
             FFTK_CASE(8)
+            FFTK_CASE(9)
+            FFTK_CASE(10)
             FFTK_CASE(11)
             FFTK_CASE(13)
             FFTK_CASE(16)
@@ -195,7 +198,10 @@ int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint3
     {
         if(p->nthreads == 0 || (p->nthreads & 63) || lds_bytes > MAX_LDS_BYTES || grid == 0)
             return (int)hipErrorInvalidValue;
-        return fftrt_launch_fast_tile(p, precision, vec, grid, lds_bytes, stream);
+        int rc = fftrt_launch_fast_tile(p, precision, vec, grid, lds_bytes, stream);
+        if(rc != FFTRT_NO_FAST_VARIANT)
+            return rc;
+        // no compiled variant for this access mode: the generic kernel runs the same schedule
     }
     if(p->nthreads == 0 || p->nthreads > 512 || (p->nthreads & 63) || lds_bytes > MAX_LDS_BYTES
        || grid == 0)

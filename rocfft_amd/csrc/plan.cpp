@@ -334,15 +334,39 @@ static uint32_t lds_pitch(uint32_t n)
     return p | 1u; // odd, so neighbouring transforms start in different banks
 }
 
+// Pass schedule of a tile kernel for length n: the one of the compile-time-schedule kernel
+// when the runtime has one for this length, else the planner's own factorisation.  Returns
+// the threads per transform (0: no schedule); *fast tells which kind it is.
+static uint32_t kernel_schedule(uint64_t n, int precision, std::vector<uint32_t>& radix, bool* fast)
+{
+    radix.clear();
+    if(fast)
+        *fast = false;
+    if(n < 1 || n > 65536)
+        return 0;
+    if(g_use_fast)
+    {
+        uint32_t fr[FFTK_MAX_PASSES] = {0}, fnf = 0;
+        uint32_t tpt = fftrt_fast_schedule(precision, (uint32_t)n, fr, &fnf);
+        if(tpt && fnf >= 1 && fnf <= 4)
+        {
+            radix.assign(fr, fr + fnf);
+            if(fast)
+                *fast = true;
+            return tpt;
+        }
+    }
+    if(!factorize(n, radix))
+        return 0;
+    return threads_per_transform(n, radix);
+}
+
 // can a single tile kernel transform length n (one transform per workgroup at least)?
 static bool single_kernel_length(uint64_t n, size_t elem_bytes)
 {
-    if(n < 1 || n > 65536)
-        return false;
     std::vector<uint32_t> radix;
-    if(!factorize(n, radix))
-        return false;
-    if(threads_per_transform(n, radix) > MAX_THREADS)
+    uint32_t              T = kernel_schedule(n, elem_bytes == 16 ? 1 : 0, radix, nullptr);
+    if(T == 0 || T > MAX_THREADS)
         return false;
     return (size_t)lds_pitch((uint32_t)n) * elem_bytes <= LDS_HARD_BYTES;
 }
@@ -485,7 +509,9 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     memset(&k, 0, sizeof(k));
     k.n = s.n;
     std::vector<uint32_t> radix;
-    if(!factorize(s.n, radix))
+    bool                  have_fast = false;
+    const uint32_t        sched_T   = kernel_schedule(s.n, precision, radix, &have_fast);
+    if(sched_T == 0)
         fail("length has no kernel factorisation");
     k.nf         = (uint32_t)radix.size();
     uint32_t cum = 1;
@@ -587,14 +613,14 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     }
 
     // work split
-    k.T        = threads_per_transform(s.n, radix);
+    k.T        = sched_T;
     k.padshift = PADSHIFT;
     k.pitch    = lds_pitch(s.n);
     if(k.T > MAX_THREADS)
         fail("transform too long for one workgroup");
     // a kernel compiled for exactly this pass schedule, when there is one
     uint32_t max_threads = MAX_THREADS;
-    uint32_t fast_tpt    = g_use_fast ? fftrt_fast_tpt(precision, k.n, k.radix, k.nf) : 0;
+    uint32_t fast_tpt    = have_fast ? sched_T : 0;
     if(fast_tpt)
     {
         k.fast      = 1;
@@ -709,8 +735,6 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         if(s.load_op == FFTK_LOAD_C2R_PRE && (k.flags & (FFTK_F_CHIRP_LOAD | FFTK_F_CONV)))
             ops_ok = false;
         if(s.store_op == FFTK_STORE_R2C_POST && (k.flags & (FFTK_F_CHIRP_STORE | FFTK_F_TWIDDLE_STORE)))
-            ops_ok = false;
-        if((s.load_op == FFTK_LOAD_C2R_PRE || s.store_op == FFTK_STORE_R2C_POST) && (k.n & 1))
             ops_ok = false;
         if(k.fast && vec && ops_ok && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
         {
@@ -834,22 +858,23 @@ static bool factorize(uint64_t n, std::vector<uint32_t>& radix);
 static bool fast_kernel_exists(uint64_t n, size_t esize)
 {
     std::vector<uint32_t> radix;
-    if(!factorize(n, radix) || radix.size() > FFTK_MAX_PASSES)
-        return false;
-    return fftrt_fast_tpt(esize == 16 ? 1 : 0, (uint32_t)n, radix.data(), (uint32_t)radix.size()) != 0;
+    bool                  fast = false;
+    kernel_schedule(n, esize == 16 ? 1 : 0, radix, &fast);
+    return fast;
 }
 
 // Will emit_dim transform a plain complex dimension of length n with one tile pass?
 static bool plain_dim_is_single(uint64_t n, bool column, size_t esize)
 {
     bool single = column ? column_kernel_length(n, esize) : single_kernel_length(n, esize);
-    // Power-of-two lengths above 4096 have no compile-time-schedule kernel; two passes of those
-    // kernels beat one pass of the run-time-schedule kernel, so split them when that is possible.
-    if(single && g_use_fast && n > 4096 && (n & (n - 1)) == 0 && !fast_kernel_exists(n, esize))
+    // Lengths above 4096 mostly have no compile-time-schedule kernel; two passes of those
+    // kernels beat one pass of the run-time-schedule kernel, so split them when both factors
+    // have one.
+    if(single && g_use_fast && n > 4096 && !fast_kernel_exists(n, esize))
     {
         uint64_t a1, a0;
         split_length(n, esize, column, a1, a0);
-        if(a1 != 0)
+        if(a1 != 0 && ((n & (n - 1)) == 0 || (fast_kernel_exists(a1, esize) && fast_kernel_exists(a0, esize))))
             single = false;
     }
     return single;

@@ -9,6 +9,7 @@
 // operations numerically without a GPU.  The product library never contains or
 // loads this file.
 #include "gpu_rt.h"
+#include "fast_core.h"
 #include "tile_core.h"
 #include <cstdlib>
 #include <cstring>
@@ -43,8 +44,11 @@ void emu_passes(const fftk_params& p, typename cplx_of<T>::type* lds)
                     EMU_CASE(3)
                     EMU_CASE(4)
                     EMU_CASE(5)
+                    EMU_CASE(6)
                     EMU_CASE(7)
                     EMU_CASE(8)
+                    EMU_CASE(9)
+                    EMU_CASE(10)
                     EMU_CASE(11)
                     EMU_CASE(13)
                     EMU_CASE(16)
@@ -141,9 +145,36 @@ int fftrt_stream_capturing(void*)
     return 0;
 }
 
-// the emulation only has the generic kernel
-uint32_t fftrt_fast_tpt(int, uint32_t, const uint32_t*, uint32_t)
+// The emulation only has the generic kernel, but it reports the pass schedules of the
+// compile-time-schedule kernels, so that the planner makes the same plans as on the GPU and
+// the generic kernel gets exercised on those schedules.
+namespace
 {
+struct EmuSched
+{
+    uint32_t n, radix[4], tpt[2]; // threads per transform in single, double precision
+};
+#define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD) \
+    {N, {A, B, C, D}, {(uint32_t)FastCfg<N, A, B, C, D, TTF>::TPT, (uint32_t)FastCfg<N, A, B, C, D, TTD>::TPT}},
+const EmuSched g_sched[] = {
+#include "fast_schedules.h"
+};
+#undef FAST_SCHED
+} // namespace
+
+uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* radix, uint32_t* nf)
+{
+    for(const EmuSched& e : g_sched)
+    {
+        if(e.n != n)
+            continue;
+        uint32_t cnt = 0;
+        for(uint32_t i = 0; i < 4; ++i)
+            if(e.radix[i] > 1)
+                radix[cnt++] = e.radix[i];
+        *nf = cnt;
+        return e.tpt[precision ? 1 : 0];
+    }
     return 0;
 }
 

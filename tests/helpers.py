@@ -241,3 +241,17 @@ def check(lib, backend, kind, lengths, batch, precision, **kw):
     tol = tolerance(precision)
     assert l2 <= tol and linf <= tol, (kind, lengths, batch, precision, kw, l2, linf)
     return l2, linf
+
+
+def fast_schedules():
+    """[(n, radices, threads single, threads double)] from the list of compile-time-schedule
+    kernels (rocfft_amd/csrc/fast_schedules.h); threads 0 = the fewest possible"""
+    import os
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "rocfft_amd", "csrc", "fast_schedules.h")).read()
+    out = []
+    for m in re.finditer(r"^FAST_SCHED\(([\d, ]+)\)", text, re.M):
+        v = [int(a) for a in m.group(1).split(",")]
+        out.append((v[2], [r for r in v[3:7] if r > 1], v[7], v[8]))
+    return out

@@ -57,6 +57,41 @@ def test_real_1d(gpu, n):
             H.check(lib, be, kind, [n], 2, prec, inplace=True)
 
 
+def test_every_compiled_schedule(gpu):
+    """Each length with a compile-time-schedule kernel: complex both directions, and the real
+    transforms of twice the length (whose half-length complex transform is that kernel with the
+    fused pre/post-processing, odd lengths included)."""
+    lib, be = gpu
+    for n, radix, tf, td in H.fast_schedules():
+        print("schedule", n, radix, flush=True)
+        H.check(lib, be, B.COMPLEX_FORWARD, [n], 5, B.SINGLE)
+        H.check(lib, be, B.COMPLEX_INVERSE, [n], 3, B.DOUBLE, inplace=True)
+        H.check(lib, be, B.REAL_FORWARD, [2 * n], 3, B.SINGLE)
+        H.check(lib, be, B.REAL_INVERSE, [2 * n], 3, B.DOUBLE)
+
+
+def test_compiled_schedules_in_other_layouts(gpu):
+    """Strided, planar and column uses of non-power-of-two schedules: column passes of the
+    compiled kernel, and the generic kernel on the same schedule where the layout has no
+    compiled variant."""
+    lib, be = gpu
+    K = B
+    for n in (100, 243, 1000, 3000):
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 3, K.SINGLE, in_type=K.COMPLEX_PLANAR, out_type=K.COMPLEX_PLANAR)
+        H.check(lib, be, K.COMPLEX_INVERSE, [n], 3, K.DOUBLE, in_strides=[3], in_dist=3 * n + 5, out_strides=[2],
+                out_dist=2 * n + 1)
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 8, K.SINGLE, in_strides=[8], in_dist=1, out_strides=[8], out_dist=1)
+        H.check(lib, be, K.REAL_FORWARD, [2 * n], 3, K.DOUBLE, out_type=K.HERMITIAN_PLANAR)
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 2, K.DOUBLE, scale=0.125)
+    for lengths in ([100, 100], [60, 90], [9, 10, 6], [1000, 12], [12, 1000], [360, 360]):
+        for kind in (K.COMPLEX_FORWARD, K.REAL_FORWARD, K.REAL_INVERSE):
+            H.check(lib, be, kind, lengths, 2, K.SINGLE)
+            H.check(lib, be, kind, lengths, 2, K.DOUBLE, inplace=(kind == K.COMPLEX_FORWARD))
+    for n in (5000, 6000, 9000, 10000, 6561, 100000):
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 2, K.SINGLE)
+        H.check(lib, be, K.REAL_INVERSE, [n], 2, K.DOUBLE)
+
+
 @pytest.mark.parametrize("n", [16384, 32768, 65536, 2 ** 18, 2 ** 20, 6000, 30030, 10007, 4099, 8198, 65537])
 def test_long_1d(gpu, n):
     lib, be = gpu

@@ -225,6 +225,34 @@ def test_every_tile_fits_the_hardware(emu):
                 assert lds <= 160 * 1024 and grid >= 1
 
 
+def test_compiled_schedule_list_is_consistent(emu):
+    """Every listed length has one schedule, its radices multiply to the length, the thread
+    count respects the register budget of 16 values per thread, and the planner uses it."""
+    rows = H.fast_schedules()
+    assert len(rows) == len({r[0] for r in rows}) and len(rows) > 200
+    for n, radix, tf, td in rows:
+        assert int(np.prod(radix)) == n and 1 <= len(radix) <= 4
+        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 16) for r in radix)
+        need = max(-(-(n // r) // (16 // r)) for r in radix)
+        for t in (tf, td):
+            assert t == 0 or need <= t <= 512
+    for n, radix, tf, td in rows[::7]:
+        st, text, _ = emu.describe(B.NOTINPLACE, 0, 0, [n], 4)
+        assert st == 0
+        assert ("radix " + "x".join(map(str, radix)) + " ") in text, (n, text)
+
+
+# the emulation runs the generic kernel on the schedules of the compiled kernels, composite
+# radices 6, 9 and 10 included
+@pytest.mark.parametrize("n", [6, 9, 10, 12, 18, 36, 60, 81, 90, 100, 120, 125, 243, 250, 360, 480, 729,
+                               1000, 1536, 2187, 3000, 3645, 4000, 4032])
+def test_compiled_schedules_on_the_generic_kernel(emu, n):
+    H.check(emu, HOST, B.COMPLEX_FORWARD, [n], 3, B.SINGLE)
+    H.check(emu, HOST, B.COMPLEX_INVERSE, [n], 2, B.DOUBLE, inplace=True)
+    H.check(emu, HOST, B.REAL_FORWARD, [2 * n], 2, B.DOUBLE)
+    H.check(emu, HOST, B.REAL_INVERSE, [2 * n], 2, B.SINGLE)
+
+
 # ------------------------------------------------------------------ numerics through the emulation
 SMALL_1D = [1, 2, 3, 4, 5, 7, 8, 9, 16, 25, 30, 49, 64, 100, 128, 256, 512, 1024, 2048, 4096, 8192,
             11, 13, 17, 19, 97, 121, 169, 1001, 2310]
