@@ -22,11 +22,12 @@ namespace
 
 // MODE 0: scalar accesses, every fused operation; 1: vector accesses, every fused operation;
 // 2: the lean path (vector accesses, interleaved complex on both sides)
-// workgroups have up to 256 threads, or 512 when one transform alone needs more than 256
+// Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
+// their tile rows wide); no kernel here needs more than the 256 registers that leaves a thread.
 template <typename Cfg>
 constexpr int fast_block_limit()
 {
-    return Cfg::TPT > 256 ? 512 : 256;
+    return 512;
 }
 
 template <typename T, typename Cfg, int MODE>
@@ -203,7 +204,7 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
                                       size_t lds_bytes, void* stream)
 {
     const FastEntry* e = find_fast(precision, p->n);
-    if(!e || p->T != e->tpt || p->nthreads > (e->tpt > 256 ? 512u : 256u) || p->padshift != 4)
+    if(!e || p->T != e->tpt || p->nthreads > 512u || p->padshift != 4)
         return (int)hipErrorInvalidValue;
     uint32_t cnt = 0;
     for(uint32_t i = 0; i < 4; ++i)

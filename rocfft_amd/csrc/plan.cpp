@@ -21,6 +21,7 @@ namespace fftamd
 static const size_t   LDS_SOFT_BYTES = 64 * 1024;  // preferred tile footprint (two workgroups per CU)
 static const size_t   LDS_HARD_BYTES = 160 * 1024; // LDS of one CU
 static const size_t   LDS_COL_BYTES  = 80 * 1024;  // a column tile may grow to this to keep its rows wide
+static const size_t   LDS_WIDE_BYTES = 140 * 1024; // ... and to this when the alternative is a second pass
 static const uint32_t MAX_THREADS    = 512;
 static const uint32_t PADSHIFT       = 4;
 // a strided ("column") pass wants at least this many bytes contiguous per row of its tile
@@ -387,6 +388,35 @@ static uint32_t floor_pow2(uint64_t v)
         p *= 2;
     return p;
 }
+// widest tile (transforms per workgroup) a strided pass over length n can have: bounded by
+// the 512 threads of a workgroup and by LDS_WIDE_BYTES
+static uint32_t widest_column_tile(uint64_t n, size_t elem_bytes)
+{
+    std::vector<uint32_t> radix;
+    uint32_t              T = kernel_schedule(n, elem_bytes == 16 ? 1 : 0, radix, nullptr);
+    if(T == 0 || T > MAX_THREADS)
+        return 0;
+    size_t per_tile = (size_t)lds_pitch((uint32_t)n) * elem_bytes;
+    if(per_tile > LDS_WIDE_BYTES)
+        return 0;
+    return std::min(floor_pow2(MAX_THREADS / T), floor_pow2(LDS_WIDE_BYTES / per_tile));
+}
+
+// May a whole strided dimension of length n (strides is/os scalars between its elements) run
+// as one strided pass even though its tile cannot keep COL_RUN_BYTES per row?  Measured on
+// MI355X: one pass with 64-byte rows beats two passes, and so does one with 32-byte rows
+// unless the stride is a multiple of 512 bytes (rows a power-of-two stride apart alias onto
+// the same HBM channels).
+static bool narrow_column_ok(uint64_t n, size_t elem_bytes, int64_t is, int64_t os)
+{
+    if(is <= 0 || os <= 0)
+        return false;
+    const size_t run     = (size_t)widest_column_tile(n, elem_bytes) * elem_bytes;
+    const size_t scalar  = elem_bytes / 2;
+    const bool   aligned = ((size_t)is * scalar) % 512 == 0 || ((size_t)os * scalar) % 512 == 0;
+    return run >= 64 || (!aligned && run >= 32);
+}
+
 static uint32_t ceil_pow2(uint64_t v)
 {
     uint32_t p = 1;
@@ -625,7 +655,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     {
         k.fast      = 1;
         k.T         = fast_tpt;
-        max_threads = fast_tpt > 256 ? 512 : 256;
+        // a strided pass may use the larger workgroup to keep its tile rows wide
+        max_threads = (fast_tpt > 256 || k.in_fast_tile || k.out_fast_tile) ? 512 : 256;
     }
     size_t   per_tile  = (size_t)k.pitch * esize;
     uint32_t w_threads = floor_pow2(max_threads / k.T);
@@ -641,6 +672,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         uint32_t w_run = (uint32_t)std::max<size_t>(1, COL_RUN_BYTES / esize);
         if(w_lds < w_run && per_tile * w_run <= LDS_COL_BYTES)
             w_lds = w_run;
+        else if(w_lds < w_run && per_tile <= LDS_WIDE_BYTES)
+            w_lds = std::max(w_lds, std::min(w_run, floor_pow2(LDS_WIDE_BYTES / per_tile)));
         W = std::min(std::min<uint32_t>(64, w_threads), std::min(w_lds, w_cap));
     }
     else
@@ -864,9 +897,11 @@ static bool fast_kernel_exists(uint64_t n, size_t esize)
 }
 
 // Will emit_dim transform a plain complex dimension of length n with one tile pass?
-static bool plain_dim_is_single(uint64_t n, bool column, size_t esize)
+// is/os: scalar strides of the dimension on both sides (0 = not known)
+static bool plain_dim_is_single(uint64_t n, bool column, size_t esize, int64_t is, int64_t os)
 {
-    bool single = column ? column_kernel_length(n, esize) : single_kernel_length(n, esize);
+    bool single = column ? (column_kernel_length(n, esize) || narrow_column_ok(n, esize, is, os))
+                         : single_kernel_length(n, esize);
     // Lengths above 4096 mostly have no compile-time-schedule kernel; two passes of those
     // kernels beat one pass of the run-time-schedule kernel, so split them when both factors
     // have one.
@@ -1016,7 +1051,7 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     blu.buf = BUF_BLU;
 
     // a pass that is not "plain" (fused real/odd handling) stays single if it fits at all
-    bool single = plain ? plain_dim_is_single(n, column, esize) : single_kernel_length(n, esize);
+    bool single = plain ? plain_dim_is_single(n, column, esize, t_is, t_os) : single_kernel_length(n, esize);
     if(single)
     {
         TileSpec s = base_spec();
@@ -1547,7 +1582,7 @@ static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t 
     for(size_t i = 0; i < rank; ++i)
         if(i != e && len[i] > 1 && (src.stride[i] < src.stride[e] || out.stride[i] < out.stride[e]))
             column = true;
-    if(!column || !smooth(n) || column_kernel_length(n, esize))
+    if(!column || !smooth(n) || plain_dim_is_single(n, true, esize, src.stride[e], out.stride[e]))
         return false;
     uint64_t n1, n0;
     split_length(n, esize, true, n1, n0);
@@ -1558,7 +1593,10 @@ static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t 
     for(size_t i = 0; i < rank; ++i)
         if(i != d && len[i] > 1 && (src.stride[i] < src.stride[d]))
             d_column = true;
-    if(!plain_dim_is_single(len[d], d_column, esize))
+    int64_t d_packed = 2; // stride of dimension d in the packed intermediate array
+    for(size_t i = 0; i < d; ++i)
+        d_packed *= (int64_t)len[i];
+    if(!plain_dim_is_single(len[d], d_column, esize, src.stride[d], d_packed))
         return false;
     if(src.io.planar || out.io.planar)
         return false;
