@@ -232,6 +232,9 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     constexpr int                     PAIRS      = (N + 1) / 2; // bins j paired with N-j (j = 0 pairs with N)
     constexpr int                     PAIR_IT    = (PAIRS + Cfg::TPT - 1) / Cfg::TPT;
     constexpr bool                    PAIR_EXACT = PAIRS % Cfg::TPT == 0;
+    // transforms whose lanes cover 16 contiguous bytes or less can go through LDS instead
+    constexpr bool                    STAGE_OK = Cfg::TPT == 1 || Cfg::TPT * sizeof(C) <= 16;
+    constexpr int                     STAGE_IT = (N + Cfg::TPT - 1) / Cfg::TPT;
     const bool                        ok   = active && (c.tile0 + w < p.tile_cnt);
     const bool                        inv  = p.dir > 0;
     const C*       src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
@@ -287,6 +290,26 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 z.y                         = (T)-2 * a.y;
                 lds[fk_addr<Cfg>(w, N / 2)] = c_swap(z);
             }
+        }
+        __syncthreads();
+        if(active)
+            fk_read<T, Cfg, 0>(lds, w, tt, r);
+        lds_busy = true;
+    }
+    else if(STAGE_OK && p.stage_io)
+    {
+        // consecutive lanes copy consecutive elements of the tile into LDS
+        const uint32_t total = p.W * N;
+#pragma unroll
+        for(int i = 0; i < STAGE_IT; ++i)
+        {
+            const uint32_t e     = tid + i * p.nthreads;
+            const uint32_t w_    = e / (uint32_t)N;
+            const uint32_t j_    = e - w_ * (uint32_t)N;
+            const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
+            C              v     = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
+            if(valid)
+                lds[fk_addr<Cfg>(w_, j_)] = inv ? c_swap(v) : v;
         }
         __syncthreads();
         if(active)
@@ -448,6 +471,35 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 o.x                            = z.x * sc;
                 o.y                            = -z.y * sc;
                 dst[(N / 2) * p.t_os_c + wo] = o;
+            }
+        }
+        return;
+    }
+
+    if(STAGE_OK && p.stage_io)
+    {
+        if(Cfg::NP > 1 || lds_busy)
+            __syncthreads();
+        if(active)
+            fk_write<T, Cfg, LAST>(lds, w, tt, r);
+        __syncthreads();
+        const uint32_t total = p.W * N;
+        const T        sc    = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
+#pragma unroll
+        for(int i = 0; i < STAGE_IT; ++i)
+        {
+            const uint32_t e     = tid + i * p.nthreads;
+            const uint32_t w_    = e / (uint32_t)N;
+            const uint32_t j_    = e - w_ * (uint32_t)N;
+            const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
+            if(valid)
+            {
+                C v = lds[fk_addr<Cfg>(w_, j_)];
+                if(out_inv)
+                    v = c_swap(v);
+                v.x *= sc;
+                v.y *= sc;
+                dst[j_ * p.t_os_c + w_ * p.w_os_c] = v;
             }
         }
         return;

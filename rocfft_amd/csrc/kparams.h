@@ -66,6 +66,9 @@ struct fftk_params
     uint32_t lean;       // fast kernel: plain interleaved complex in and out, strides below in
                          // complex elements fit 32 bits: branch-free addressing path
     uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
+    uint32_t stage_io; // lean path: move the tile between global memory and LDS with consecutive
+                       // lanes on consecutive elements (transforms too short for coalesced
+                       // register loads)
     uint32_t flags;
     int32_t  dir; // -1 forward, +1 inverse
     uint32_t load_op, store_op;

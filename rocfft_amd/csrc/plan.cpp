@@ -776,6 +776,11 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             if(in_span < (1ull << 28) && out_span < (1ull << 28))
             {
                 rec.lean_ok = true;
+                // short transforms in unit-stride rows: coalesced tile copies through LDS
+                if(!column && (k.T == 1 || ((size_t)k.T * esize <= 16 && k.n < 32)) && k.t_is == 2 && k.t_os == 2
+                   && s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_COMPLEX
+                   && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0 && k.n_in == k.n && k.n_out == k.n)
+                    k.stage_io = 1;
                 k.t_is_c    = (uint32_t)(k.t_is / 2);
                 k.t_os_c    = (uint32_t)(k.t_os / 2);
                 k.w_is_c    = (uint32_t)(k.w_is / 2);
@@ -902,14 +907,15 @@ static bool plain_dim_is_single(uint64_t n, bool column, size_t esize, int64_t i
 {
     bool single = column ? (column_kernel_length(n, esize) || narrow_column_ok(n, esize, is, os))
                          : single_kernel_length(n, esize);
-    // Lengths above 4096 mostly have no compile-time-schedule kernel; two passes of those
-    // kernels beat one pass of the run-time-schedule kernel, so split them when both factors
-    // have one.
-    if(single && g_use_fast && n > 4096 && !fast_kernel_exists(n, esize))
+    // Longer lengths without a compile-time-schedule kernel (most above 4096, 5^5 below): two
+    // passes of those kernels beat one pass of the run-time-schedule kernel, so split them
+    // when both factors have one.
+    if(single && g_use_fast && n >= 1024 && !fast_kernel_exists(n, esize))
     {
         uint64_t a1, a0;
         split_length(n, esize, column, a1, a0);
-        if(a1 != 0 && ((n & (n - 1)) == 0 || (fast_kernel_exists(a1, esize) && fast_kernel_exists(a0, esize))))
+        if(a1 != 0 && ((n > 4096 && (n & (n - 1)) == 0)
+                       || (fast_kernel_exists(a1, esize) && fast_kernel_exists(a0, esize))))
             single = false;
     }
     return single;
@@ -2053,7 +2059,7 @@ std::string ExecPlan::describe() const
                 o << " lean";
             if(k.fast)
                 o << " fast" << (k.direct_in ? " direct_in" : " staged_in")
-                  << (k.direct_out ? " direct_out" : " staged_out");
+                  << (k.direct_out ? " direct_out" : " staged_out") << (k.stage_io ? " tile_copy" : "");
         }
         else if(r.kind == PASS_BIG)
             o << " threads 1024 grid " << r.grid << " lds 135296";
