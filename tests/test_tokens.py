@@ -1,0 +1,109 @@
+"""Reference-client vocabulary: token strings (shared/fft_params.h:726-1059 of the reference)
+parsed into plans, and the rocfft-bench style command line."""
+import numpy as np
+import pytest
+
+import helpers as H
+import rocfft_amd.binding as B
+from rocfft_amd.params import FFTParams, TokenError, TOKEN_SCALE_FACTOR
+
+HOST = H.HostBackend()
+
+# the five benchmark configurations as the reference clients would name them
+CONFIG_TOKENS = [
+    "complex_forward_len_4096_single_ip_batch_1024_istride_1_CI_ostride_1_CI_idist_4096_odist_4096_ioffset_0_0_ooffset_0_0",
+    "real_forward_len_65536_single_op_batch_4096_istride_1_R_ostride_1_HI_idist_65536_odist_32769_ioffset_0_0_ooffset_0_0",
+    "real_inverse_len_65536_single_op_batch_4096_istride_1_HI_ostride_1_R_idist_32769_odist_65536_ioffset_0_0_ooffset_0_0",
+    "complex_forward_len_4096_4096_single_op_batch_8_istride_4096_1_CI_ostride_4096_1_CI_idist_16777216_odist_16777216_ioffset_0_0_ooffset_0_0",
+    "real_forward_len_512_512_512_double_op_batch_1_istride_262144_512_1_R_ostride_131584_257_1_HI_idist_134217728_odist_67371008_ioffset_0_0_ooffset_0_0",
+    "real_inverse_len_512_512_512_double_op_batch_1_istride_131584_257_1_HI_ostride_262144_512_1_R_idist_67371008_odist_134217728_ioffset_0_0_ooffset_0_0",
+    "complex_forward_len_1000003_double_op_batch_16_istride_1_CI_ostride_1_CI_idist_1000003_odist_1000003_ioffset_0_0_ooffset_0_0",
+]
+
+
+@pytest.mark.parametrize("token", CONFIG_TOKENS)
+def test_token_round_trip(token):
+    p = FFTParams.from_token(token)
+    assert p.token() == token
+    # the defaults reproduce the explicit layout of these tokens
+    q = FFTParams(p.transform_type, p.length, p.precision, p.placement, p.nbatch).validate()
+    assert q.token() == token
+
+
+def test_token_fields():
+    p = FFTParams.from_token("real_forward_len_8_6_double_ip_batch_3_istride_8_1_R_ostride_4_1_HI_idist_48_odist_24"
+                             "_ioffset_0_0_ooffset_0_0_scale")
+    assert (p.transform_type, p.length, p.precision, p.placement, p.nbatch) == (B.REAL_FORWARD, [8, 6], B.DOUBLE,
+                                                                                B.INPLACE, 3)
+    assert (p.istride, p.itype, p.ostride, p.otype) == ([8, 1], B.REAL, [4, 1], B.HERMITIAN_INTERLEAVED)
+    assert (p.idist, p.odist, p.scale_factor) == (48, 24, TOKEN_SCALE_FACTOR)
+    # in-place real defaults: rows padded to 2 (N/2 + 1) reals
+    q = FFTParams(B.REAL_FORWARD, [8, 6], B.DOUBLE, B.INPLACE, 3).validate()
+    assert (q.istride, q.idist, q.ostride, q.odist) == ([8, 1], 64, [4, 1], 32)
+    assert q.isize() == 2 * 64 + 7 * 8 + 5 + 1 and q.osize() == 2 * 32 + 7 * 4 + 3 + 1
+    p = FFTParams.from_token("complex_inverse_len_16_single_op_batch_2_istride_2_CP_ostride_1_CI_idist_40_odist_16"
+                             "_ioffset_3_5_ooffset_1_0")
+    assert (p.itype, p.ibuffers(), p.obuffers(), p.ioffset, p.ooffset) == (B.COMPLEX_PLANAR, 2, 1, [3, 5], [1, 0])
+
+
+@pytest.mark.parametrize("bad", [
+    "complex_sideways_len_8_single_ip_batch_1",
+    "complex_forward_len_8_quad_ip_batch_1",
+    "complex_forward_len_8_single_ip_batch",
+    "complex_forward_len_8_single_ip_batch_1_istride_1_CI_ostride_1_CI_idist_8_odist_8_ioffset_0_0_ooffset_0_0_CB",
+    "complex_forward_len_8_single_ip_batch_1_ifield_brick_lower_0_upper_8_stride_1_dev_0",
+    "complex_forward_len_8_single_ip_batch_1_multiGPU_2",
+])
+def test_bad_tokens_are_rejected(bad):
+    with pytest.raises(TokenError):
+        FFTParams.from_token(bad).validate()
+
+
+def run_token(lib, backend, token):
+    """executes the plan a token describes and compares with the CPU checker"""
+    p = FFTParams.from_token(token).validate()
+    rev = lambda v: list(reversed(v))
+    kw = dict(inplace=p.placement == B.INPLACE, in_type=p.itype, out_type=p.otype, in_strides=rev(p.istride),
+              in_dist=p.idist, out_strides=rev(p.ostride), out_dist=p.odist, in_offsets=p.ioffset,
+              out_offsets=p.ooffset)
+    if p.scale_factor != 1.0:
+        kw["scale"] = p.scale_factor
+    return H.check(lib, backend, p.transform_type, rev(p.length), p.nbatch, p.precision, **kw)
+
+
+SMALL_TOKENS = [
+    "complex_forward_len_4096_single_ip_batch_3_istride_1_CI_ostride_1_CI_idist_4096_odist_4096_ioffset_0_0_ooffset_0_0",
+    "real_forward_len_256_single_op_batch_4_istride_1_R_ostride_1_HI_idist_256_odist_129_ioffset_0_0_ooffset_0_0",
+    "real_inverse_len_256_double_op_batch_4_istride_1_HI_ostride_1_R_idist_129_odist_256_ioffset_0_0_ooffset_0_0",
+    "complex_forward_len_64_32_single_op_batch_2_istride_32_1_CI_ostride_32_1_CI_idist_2048_odist_2048_ioffset_0_0_ooffset_0_0",
+    "real_forward_len_8_16_32_double_op_batch_1_istride_512_32_1_R_ostride_272_17_1_HI_idist_4096_odist_2176_ioffset_0_0_ooffset_0_0",
+    "complex_inverse_len_100_double_op_batch_3_istride_2_CP_ostride_1_CI_idist_210_odist_100_ioffset_3_5_ooffset_1_0",
+    "complex_forward_len_30_double_op_batch_2_istride_1_CI_ostride_1_CI_idist_30_odist_30_ioffset_0_0_ooffset_0_0_scale",
+    "real_forward_len_20_6_single_ip_batch_2_istride_8_1_R_ostride_4_1_HI_idist_160_odist_80_ioffset_0_0_ooffset_0_0",
+    "complex_forward_len_8_1024_single_op_batch_1_istride_1_8_CI_ostride_1024_1_CI_idist_8192_odist_8192_ioffset_0_0_ooffset_0_0",
+]
+
+
+@pytest.mark.parametrize("token", SMALL_TOKENS)
+def test_tokens_through_the_emulation(emu, token):
+    run_token(emu, HOST, token)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("token", SMALL_TOKENS)
+def test_tokens_on_the_gpu(gpu_lib, token):
+    run_token(gpu_lib, H.TorchBackend(), token)
+
+
+@pytest.mark.gpu
+def test_bench_command_line(gpu_lib, capsys):
+    from rocfft_amd import bench_cli
+
+    assert bench_cli.main(["--token", SMALL_TOKENS[0], "-N", "3"]) == 0
+    assert bench_cli.main(["--length", "64", "32", "-t", "2", "--precision", "double", "-o", "-b", "2", "-N", "2"]) == 0
+    out = capsys.readouterr().out
+    lines = [l for l in out.splitlines() if l.startswith("Execution gpu time:")]
+    assert len(lines) == 2 and len(lines[0].split()) == 3 + 3 + 1 and lines[0].endswith(" ms")
+    assert sum(l.startswith("Execution gflops:") for l in out.splitlines()) == 2
+    assert "Token: real_forward_len_64_32_double_op_batch_2_istride_32_1_R_ostride_17_1_HI_idist_2048_odist_1088" in out
+    assert bench_cli.main(["--token", "complex_forward_len_8_single_ip_batch_1_multiGPU_2"]) == 2
