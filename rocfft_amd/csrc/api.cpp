@@ -13,6 +13,8 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <sstream>
 #include <string>
 #include <vector>
 
@@ -244,8 +246,102 @@ static rocfft_status make_problem(Problem& p, rocfft_result_placement placement,
 // ---------------------------------------------------------------------------
 // entry points
 
-static int  g_setup_count = 0;
-static bool g_log_plan    = false;
+static int g_setup_count = 0;
+
+// ---------------------------------------------------------------------------
+// Log layers, selected by the bits of ROCFFT_LAYER as in the reference
+// (library/src/include/logging.h:139-150): 1 trace (every API call with its arguments),
+// 2 bench (a rocfft-bench command line per plan, library/src/plan.cpp:698-726), 4 profile
+// (duration and bandwidth of every kernel of an execute, library/src/powX.cpp:855-882),
+// 8 plan (the pass list).  Each layer writes to stderr, or appends to the file named by
+// ROCFFT_LOG_TRACE_PATH / _BENCH_PATH / _PROFILE_PATH / _PLAN_PATH
+// (library/src/auxiliary.cpp:88-128).
+enum
+{
+    LOG_TRACE   = 1,
+    LOG_BENCH   = 2,
+    LOG_PROFILE = 4,
+    LOG_PLAN    = 8
+};
+static int        g_layers = 0;
+static FILE*      g_log_file[4] = {nullptr, nullptr, nullptr, nullptr};
+static std::mutex g_log_mutex;
+
+static FILE* log_stream(int layer)
+{
+    int   i = layer == LOG_TRACE ? 0 : layer == LOG_BENCH ? 1 : layer == LOG_PROFILE ? 2 : 3;
+    FILE* f = g_log_file[i];
+    return f ? f : stderr;
+}
+
+static void log_line(int layer, const std::string& text)
+{
+    std::lock_guard<std::mutex> lock(g_log_mutex);
+    FILE*                       f = log_stream(layer);
+    fputs(text.c_str(), f);
+    if(text.empty() || text.back() != '\n')
+        fputc('\n', f);
+    fflush(f);
+}
+
+// "function,key,value,key,value,..." as the reference's trace lines
+struct TraceLine
+{
+    std::ostringstream o;
+    bool               on;
+    explicit TraceLine(const char* fn)
+        : on((g_layers & LOG_TRACE) != 0)
+    {
+        if(on)
+            o << fn;
+    }
+    template <typename V>
+    TraceLine& arg(const char* key, const V& v)
+    {
+        if(on)
+            o << "," << key << "," << v;
+        return *this;
+    }
+    TraceLine& sizes(const char* key, const size_t* v, size_t n)
+    {
+        if(on)
+        {
+            o << "," << key << ",";
+            for(size_t i = 0; v && i < n; ++i)
+                o << (i ? " " : "") << v[i];
+        }
+        return *this;
+    }
+    ~TraceLine()
+    {
+        if(on)
+            log_line(LOG_TRACE, o.str());
+    }
+};
+
+static std::string bench_command(const Problem& p)
+{
+    std::ostringstream o;
+    o << "rocfft-bench --length ";
+    for(size_t d = p.rank; d-- > 0;)
+        o << p.len[d] << " ";
+    o << "-b " << p.batch << " ";
+    if(p.placement == rocfft_placement_notinplace)
+        o << "-o ";
+    o << "-t " << (int)p.type << " --precision "
+      << (p.precision == rocfft_precision_double ? "double" : p.precision == rocfft_precision_half ? "half" : "single")
+      << " --itype " << (int)p.in_type << " --otype " << (int)p.out_type << " --istride ";
+    for(size_t d = p.rank; d-- > 0;)
+        o << p.istride[d] << " ";
+    o << "--ostride ";
+    for(size_t d = p.rank; d-- > 0;)
+        o << p.ostride[d] << " ";
+    o << "--idist " << p.idist << " --odist " << p.odist << " --ioffset " << p.ioffset[0] << " "
+      << p.ioffset[1] << " --ooffset " << p.ooffset[0] << " " << p.ooffset[1];
+    if(p.has_scale)
+        o << " --scalefactor " << p.scale;
+    return o.str();
+}
 
 extern "C" {
 
@@ -253,13 +349,24 @@ rocfft_status rocfft_setup(void)
 {
     ++g_setup_count;
     const char* layer = getenv("ROCFFT_LAYER");
-    // bit 3 of ROCFFT_LAYER asks for the plan log (reference logging.h:139-150)
-    g_log_plan = layer && (atoi(layer) & 8);
+    g_layers          = layer ? (int)strtol(layer, nullptr, 0) : 0;
+    static const char* const path_vars[4]
+        = {"ROCFFT_LOG_TRACE_PATH", "ROCFFT_LOG_BENCH_PATH", "ROCFFT_LOG_PROFILE_PATH", "ROCFFT_LOG_PLAN_PATH"};
+    for(int i = 0; i < 4; ++i)
+    {
+        const char* path = getenv(path_vars[i]);
+        if((g_layers & (1 << i)) && path && *path && !g_log_file[i])
+            g_log_file[i] = fopen(path, "a");
+    }
+    TraceLine t(__func__);
     return rocfft_status_success;
 }
 
 rocfft_status rocfft_cleanup(void)
 {
+    {
+        TraceLine t(__func__);
+    }
     if(g_setup_count > 0)
         --g_setup_count;
     table_cache_clear();
@@ -274,11 +381,21 @@ rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement plac
     if(!plan)
         return rocfft_status_failure;
     *plan = nullptr;
+    TraceLine(__func__)
+        .arg("placement", (int)placement)
+        .arg("transform_type", (int)transform_type)
+        .arg("precision", (int)precision)
+        .arg("dimensions", dimensions)
+        .sizes("lengths", lengths, dimensions <= 3 ? dimensions : 0)
+        .arg("number_of_transforms", number_of_transforms)
+        .arg("description", (const void*)description);
     try
     {
         rocfft_plan_t* p  = new rocfft_plan_t;
         rocfft_status  st = make_problem(p->prob, placement, transform_type, precision, dimensions,
                                         lengths, number_of_transforms, description);
+        if(st == rocfft_status_success && (g_layers & LOG_BENCH))
+            log_line(LOG_BENCH, bench_command(p->prob));
         if(st == rocfft_status_success)
         {
             int ndev = 0;
@@ -300,8 +417,8 @@ rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement plac
             delete p;
             return st;
         }
-        if(g_log_plan)
-            fputs(p->exec.describe().c_str(), stderr);
+        if(g_layers & LOG_PLAN)
+            log_line(LOG_PLAN, p->exec.describe());
         *plan = p;
         return rocfft_status_success;
     }
@@ -381,6 +498,32 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
 rocfft_status rocfft_execute(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
                              rocfft_execution_info info)
 {
+    TraceLine(__func__)
+        .arg("plan", (const void*)plan)
+        .arg("in_buffer", in_buffer ? in_buffer[0] : nullptr)
+        .arg("out_buffer", out_buffer ? out_buffer[0] : nullptr)
+        .arg("info", (const void*)info);
+    // the profile layer times every kernel with events and waits for them, as the reference's
+    // does; it is skipped while the stream is being captured
+    if((g_layers & LOG_PROFILE) && plan && !fftrt_stream_capturing(info ? info->stream : nullptr))
+    {
+        std::vector<float> ms(plan->exec.passes.size() + 1, 0.0f);
+        rocfft_status      st = execute_impl(plan, in_buffer, out_buffer, info, ms.data());
+        if(st != rocfft_status_success)
+            return st;
+        const double peak = 8000.0; // GB/s, HBM3E of MI355X
+        for(size_t i = 0; i < plan->exec.passes.size(); ++i)
+        {
+            const PassRec&     r  = plan->exec.passes[i];
+            const double       bw = ms[i] > 0 ? r.bytes_rw / (ms[i] * 1e6) : 0.0;
+            std::ostringstream o;
+            o << "TransformPowX,scheme," << r.note << ",duration_ms," << ms[i] << ",total_size_bytes,"
+              << (uint64_t)r.bytes_rw << ",exec_GB_s," << bw << ",max_mem_GB_s," << peak
+              << ",bw_efficiency_pct," << 100.0 * bw / peak << ",kernel_index," << i;
+            log_line(LOG_PROFILE, o.str());
+        }
+        return st;
+    }
     return execute_impl(plan, in_buffer, out_buffer, info, nullptr);
 }
 
@@ -419,6 +562,7 @@ rocfft_status rocfft_amd_plan_get_pass_info(const rocfft_plan plan, size_t index
 
 rocfft_status rocfft_plan_destroy(rocfft_plan plan)
 {
+    TraceLine(__func__).arg("plan", (const void*)plan);
     delete plan;
     return rocfft_status_success;
 }
@@ -426,6 +570,7 @@ rocfft_status rocfft_plan_destroy(rocfft_plan plan)
 rocfft_status rocfft_plan_description_set_scale_factor(rocfft_plan_description description,
                                                        const double            scale_factor)
 {
+    TraceLine(__func__).arg("description", (const void*)description).arg("scale", scale_factor);
     if(!description)
         return rocfft_status_failure;
     if(!std::isfinite(scale_factor))
@@ -447,6 +592,16 @@ rocfft_status rocfft_plan_description_set_data_layout(rocfft_plan_description de
                                                       const size_t*           out_strides,
                                                       const size_t            out_distance)
 {
+    TraceLine(__func__)
+        .arg("description", (const void*)description)
+        .arg("in_array_type", (int)in_array_type)
+        .arg("out_array_type", (int)out_array_type)
+        .sizes("in_offsets", in_offsets, 2)
+        .sizes("out_offsets", out_offsets, 2)
+        .sizes("in_strides", in_strides, in_strides_size <= 3 ? in_strides_size : 0)
+        .arg("in_distance", in_distance)
+        .sizes("out_strides", out_strides, out_strides_size <= 3 ? out_strides_size : 0)
+        .arg("out_distance", out_distance);
     if(!description)
         return rocfft_status_failure;
     auto planar = [](rocfft_array_type t) {
@@ -553,6 +708,7 @@ rocfft_status rocfft_plan_description_add_outfield(rocfft_plan_description descr
 
 rocfft_status rocfft_plan_get_work_buffer_size(const rocfft_plan plan, size_t* size_in_bytes)
 {
+    TraceLine(__func__).arg("plan", (const void*)plan);
     if(!plan || !size_in_bytes)
         return rocfft_status_failure;
     *size_in_bytes = plan->exec.work_bytes();
@@ -570,6 +726,7 @@ rocfft_status rocfft_plan_get_print(const rocfft_plan plan)
 
 rocfft_status rocfft_plan_description_create(rocfft_plan_description* description)
 {
+    TraceLine(__func__).arg("description", (const void*)description);
     if(!description)
         return rocfft_status_failure;
     *description = new rocfft_plan_description_t;
@@ -577,12 +734,14 @@ rocfft_status rocfft_plan_description_create(rocfft_plan_description* descriptio
 }
 rocfft_status rocfft_plan_description_destroy(rocfft_plan_description description)
 {
+    TraceLine(__func__).arg("description", (const void*)description);
     delete description;
     return rocfft_status_success;
 }
 
 rocfft_status rocfft_execution_info_create(rocfft_execution_info* info)
 {
+    TraceLine(__func__).arg("info", (const void*)info);
     if(!info)
         return rocfft_status_failure;
     *info = new rocfft_execution_info_t;
@@ -590,6 +749,7 @@ rocfft_status rocfft_execution_info_create(rocfft_execution_info* info)
 }
 rocfft_status rocfft_execution_info_destroy(rocfft_execution_info info)
 {
+    TraceLine(__func__).arg("info", (const void*)info);
     delete info;
     return rocfft_status_success;
 }
@@ -597,6 +757,7 @@ rocfft_status rocfft_execution_info_destroy(rocfft_execution_info info)
 rocfft_status rocfft_execution_info_set_work_buffer(rocfft_execution_info info, void* work_buffer,
                                                     const size_t size_in_bytes)
 {
+    TraceLine(__func__).arg("info", (const void*)info).arg("work_buffer", (const void*)work_buffer).arg("size_in_bytes", size_in_bytes);
     if(!info)
         return rocfft_status_failure;
     if(!work_buffer)
@@ -608,6 +769,7 @@ rocfft_status rocfft_execution_info_set_work_buffer(rocfft_execution_info info, 
 
 rocfft_status rocfft_execution_info_set_stream(rocfft_execution_info info, void* stream)
 {
+    TraceLine(__func__).arg("info", (const void*)info).arg("stream", (const void*)stream);
     if(!info)
         return rocfft_status_failure;
     info->stream = stream;

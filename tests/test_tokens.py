@@ -107,3 +107,39 @@ def test_bench_command_line(gpu_lib, capsys):
     assert sum(l.startswith("Execution gflops:") for l in out.splitlines()) == 2
     assert "Token: real_forward_len_64_32_double_op_batch_2_istride_32_1_R_ostride_17_1_HI_idist_2048_odist_1088" in out
     assert bench_cli.main(["--token", "complex_forward_len_8_single_ip_batch_1_multiGPU_2"]) == 2
+
+
+def test_log_layers(tmp_path):
+    """ROCFFT_LAYER bits 1/2/4/8 = trace, bench, profile and plan logs, each to the file its
+    ROCFFT_LOG_*_PATH variable names (reference library/src/auxiliary.cpp:88-128); the bench log
+    holds a command line that the rocfft-bench style parser reads back."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, ROCFFT_LAYER="15")
+    for name in ("TRACE", "BENCH", "PROFILE", "PLAN"):
+        env["ROCFFT_LOG_%s_PATH" % name] = str(tmp_path / (name.lower() + ".log"))
+    code = ("import sys; sys.path[:0] = [%r, %r]\n"
+            "import helpers as H, rocfft_amd.binding as B\n"
+            "emu = B.Library(%r); emu.setup()\n"
+            "H.check(emu, H.HostBackend(), B.REAL_FORWARD, [64, 8], 2, B.DOUBLE, scale=0.5)\n"
+            % (root, os.path.join(root, "tests"), os.path.join(root, "tests", "emu", "librocfft_amd_emu.so")))
+    subprocess.check_call([sys.executable, "-c", code], env=env)
+    trace = (tmp_path / "trace.log").read_text().splitlines()
+    assert trace[0] == "rocfft_setup"
+    assert any(l.startswith("rocfft_plan_create,placement,1,transform_type,2,precision,1,dimensions,2,lengths,64 8,"
+                            "number_of_transforms,2,") for l in trace)
+    assert any(l.startswith("rocfft_execute,plan,") for l in trace)
+    bench = (tmp_path / "bench.log").read_text().strip()
+    assert bench == ("rocfft-bench --length 8 64 -b 2 -o -t 2 --precision double --itype 2 --otype 3 --istride 64 1 "
+                     "--ostride 33 1 --idist 512 --odist 264 --ioffset 0 0 --ooffset 0 0 --scalefactor 0.5")
+    from rocfft_amd import bench_cli
+    p = bench_cli.params_from_args(bench_cli.parse(bench.split()[1:])).validate()
+    assert p.token() == ("real_forward_len_8_64_double_op_batch_2_istride_64_1_R_ostride_33_1_HI_idist_512_odist_264"
+                         "_ioffset_0_0_ooffset_0_0_scale")
+    profile = (tmp_path / "profile.log").read_text().splitlines()
+    assert len(profile) == 2 and all(l.startswith("TransformPowX,scheme,") and ",kernel_index," in l for l in profile)
+    plan = (tmp_path / "plan.log").read_text()
+    assert plan.startswith("plan: 2 passes, precision double")
