@@ -79,6 +79,12 @@ __global__ __launch_bounds__(256) void real_post_kernel(const fftk_real_params p
 }
 
 template <typename T>
+__global__ __launch_bounds__(256) void row_copy_kernel(const fftk_copy_params p)
+{
+    copy_elem<T>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
+}
+
+template <typename T>
 __global__ __launch_bounds__(256) void real_pre_kernel(const fftk_real_params p)
 {
     real_pre_elem<T>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
@@ -226,6 +232,19 @@ int fftrt_launch_real_post(const struct fftk_real_params* p, int precision, void
         hipLaunchKernelGGL(real_post_kernel<float>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
     else
         hipLaunchKernelGGL(real_post_kernel<double>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
+    return (int)hipGetLastError();
+}
+
+int fftrt_launch_copy(const struct fftk_copy_params* p, int precision, void* stream)
+{
+    uint64_t total = (uint64_t)p->cnt * p->rows0 * p->rows1 * p->rows2;
+    uint64_t grid  = (total + 255) / 256;
+    if(grid == 0 || grid >= (1ull << 31))
+        return (int)hipErrorInvalidValue;
+    if(precision == 0)
+        hipLaunchKernelGGL(row_copy_kernel<float>, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, *p);
+    else
+        hipLaunchKernelGGL(row_copy_kernel<double>, dim3((uint32_t)grid), dim3(256), 0, (hipStream_t)stream, *p);
     return (int)hipGetLastError();
 }
 

@@ -118,6 +118,29 @@ struct fftk_real_params
     uint32_t    use_scale;
 };
 
+// element-wise row copy between array kinds: real -> complex, complex -> real, Hermitian half
+// -> full conjugate-symmetric row, complex row -> its first elements.  The slow path of
+// odd-length real transforms too long for one kernel runs a complex transform between two
+// of these.
+struct fftk_copy_params
+{
+    uint32_t    cnt;         // elements written per row
+    uint32_t    mirror_from; // source index j >= mirror_from reads element mirror_n - j, conjugated
+    uint32_t    mirror_n;    //   (mirror_from = 0: no mirroring)
+    uint32_t    src_real;    // the source holds real values (imaginary part reads as zero)
+    uint32_t    dst_real;    // only the real part is written
+    uint32_t    zero_im0;    // the imaginary part of source element 0 reads as zero
+    uint32_t    rows0, rows1, rows2;
+    int64_t     s_s, s_r0, s_r1, s_r2; // source element stride and row strides, in scalars
+    int64_t     d_s, d_r0, d_r1, d_r2;
+    const void* s0; // real parts
+    const void* s1; // imaginary parts
+    void*       d0;
+    void*       d1;
+    double      scale;
+    uint32_t    use_scale;
+};
+
 // one-workgroup 32768-point single-precision transform (big_kernels.hip)
 struct fftk_big_params
 {

@@ -829,6 +829,10 @@ struct Builder
     {
         plan->tmp_elems = std::max(plan->tmp_elems, elems);
     }
+    void need_cpx(size_t elems)
+    {
+        plan->cpx_elems = std::max(plan->cpx_elems, elems);
+    }
     void need_blu(size_t elems)
     {
         plan->blu_elems = std::max(plan->blu_elems, elems);
@@ -1212,13 +1216,18 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     if(M >= (1ull << 31))
         fail("length too large");
     bool     conj_chirp = dir > 0;
-    TablePtr chirp      = chirp_table(N, b.precision, b.dry);
-    double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
-    uint32_t cflag      = conj_chirp ? FFTK_F_CHIRP_CONJ : 0;
     // the whole convolution in one workgroup when M fits; strided data must keep a wide tile
     bool one = column ? column_kernel_length(M, esize) : single_kernel_length(M, esize);
     if(!one && column && single_kernel_length(M, esize) && M <= 4096)
         one = true;
+    // (checked before any table is computed: a chirp of 10^8 entries takes a minute)
+    if(!one && (ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out))
+        fail("odd-length real transforms of this size are not implemented");
+    if(!one && !single_kernel_length(M / 4096, esize))
+        fail("Bluestein length too large");
+    TablePtr chirp      = chirp_table(N, b.precision, b.dry);
+    double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
+    uint32_t cflag      = conj_chirp ? FFTK_F_CHIRP_CONJ : 0;
     if(one)
     {
         TablePtr bs = bluestein_spectrum(b, N, M, 0, 0, conj_chirp);
@@ -1514,6 +1523,95 @@ static void emit_big(Builder& b, uint32_t mode, const std::vector<Other>& others
     rec.note     = names[mode];
     rec.bytes_rw = lines * (mode == 0 ? 2.0 * 32768 * 8 : (65536.0 * 4 + 32769.0 * 8));
     b.plan->passes.push_back(rec);
+}
+
+// element-wise copy of `cnt` elements per row between two array kinds (fftk_copy_params)
+static void emit_copy(Builder& b, uint32_t cnt, const std::vector<Other>& rows, int64_t s_s, const IoRef& src,
+                      int64_t d_s, const IoRef& dst, const fftk_copy_params& proto, const char* what)
+{
+    if(rows.size() > 3)
+        fail("too many dimensions");
+    PassRec rec;
+    rec.kind = PASS_COPY;
+    memset(&rec.kp, 0, sizeof(rec.kp));
+    fftk_copy_params& c = rec.cp;
+    c                   = proto;
+    c.cnt               = cnt;
+    c.rows0 = c.rows1 = c.rows2 = 1;
+    uint32_t* rc[3]             = {&c.rows0, &c.rows1, &c.rows2};
+    int64_t*  ss[3]             = {&c.s_r0, &c.s_r1, &c.s_r2};
+    int64_t*  ds[3]             = {&c.d_r0, &c.d_r1, &c.d_r2};
+    double    rowsn             = 1;
+    for(size_t i = 0; i < rows.size(); ++i)
+    {
+        *rc[i] = rows[i].cnt;
+        *ss[i] = rows[i].is;
+        *ds[i] = rows[i].os;
+        rowsn *= rows[i].cnt;
+    }
+    c.s_s   = s_s;
+    c.d_s   = d_s;
+    rec.src = src;
+    rec.dst = dst;
+    rec.note     = dims_note(what, cnt);
+    rec.bytes_rw = rowsn * cnt * (double)((c.src_real ? 1 : 2) + (c.dst_real ? 1 : 2)) * (b.precision ? 8 : 4);
+    b.plan->passes.push_back(rec);
+}
+
+// Odd-length real transform whose length needs more than one kernel: the rows are copied
+// into a complex scratch array (the reference's CS_REAL_TRANSFORM_USING_CMPLX scheme,
+// library/src/tree_node_real.cpp:115-206), transformed there as complex data, and copied out.
+// `lines`: the other dimensions and the batch, is = stride on the real side, os = stride on
+// the Hermitian side.
+static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const std::vector<Other>& others,
+                     const IoRef& src, const IoRef& dst, int dir, const DimOps& ops);
+
+static void emit_odd_real_via_complex(Builder& b, bool forward, uint64_t n, const std::vector<Other>& lines,
+                                      int64_t real_stride, const IoRef& real_io, int64_t herm_stride,
+                                      const IoRef& herm_io, double scale, bool has_scale)
+{
+    const uint64_t h = n / 2 + 1;
+    // packed complex rows in the scratch region
+    std::vector<Other> packed, in_rows, out_rows;
+    int64_t            st = 2 * (int64_t)n;
+    uint64_t           total = n;
+    for(const Other& o : lines)
+    {
+        packed.push_back({o.cnt, st, st});
+        in_rows.push_back({o.cnt, forward ? o.is : o.os, st});
+        out_rows.push_back({o.cnt, st, forward ? o.os : o.is});
+        st *= o.cnt;
+        total *= o.cnt;
+    }
+    b.need_cpx(total);
+    IoRef cpx;
+    cpx.buf = BUF_CPX;
+    fftk_copy_params proto;
+    memset(&proto, 0, sizeof(proto));
+    if(forward)
+    {
+        proto.src_real = 1;
+        emit_copy(b, (uint32_t)n, in_rows, real_stride, real_io, 2, cpx, proto, "real rows to complex scratch");
+        emit_dim(b, n, 2, 2, packed, cpx, cpx, -1, DimOps());
+        memset(&proto, 0, sizeof(proto));
+        proto.scale     = scale;
+        proto.use_scale = has_scale ? 1 : 0;
+        emit_copy(b, (uint32_t)h, out_rows, 2, cpx, herm_stride, herm_io, proto, "first bins to Hermitian rows");
+    }
+    else
+    {
+        proto.mirror_from = (uint32_t)h;
+        proto.mirror_n    = (uint32_t)n;
+        proto.zero_im0    = 1;
+        emit_copy(b, (uint32_t)n, in_rows, herm_stride, herm_io, 2, cpx, proto,
+                  "Hermitian rows to full complex scratch");
+        emit_dim(b, n, 2, 2, packed, cpx, cpx, +1, DimOps());
+        memset(&proto, 0, sizeof(proto));
+        proto.dst_real  = 1;
+        proto.scale     = scale;
+        proto.use_scale = has_scale ? 1 : 0;
+        emit_copy(b, (uint32_t)n, out_rows, 2, cpx, real_stride, real_io, proto, "real parts to real rows");
+    }
 }
 
 // standalone even-length post/pre pass over natural-order rows
@@ -1814,7 +1912,18 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                     ops.scale     = p.scale;
                     ops.has_scale = p.has_scale;
                 }
-                emit_dim(b, n0, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, -1, ops);
+                const size_t mark = plan.passes.size();
+                try
+                {
+                    emit_dim(b, n0, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, -1, ops);
+                }
+                catch(const PlanError&)
+                {
+                    // too long for the fused real load: through a complex scratch copy
+                    plan.passes.resize(mark);
+                    emit_odd_real_via_complex(b, true, n0, oth, rv.stride[0], rv.io, hv.stride[0], hv.io,
+                                              p.scale, last0 && p.has_scale);
+                }
             }
             for(size_t d = 1; d < p.rank; ++d)
             {
@@ -1882,7 +1991,20 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
             ops.n_in            = (uint32_t)n0;
             ops.scale           = p.scale;
             ops.has_scale       = p.has_scale;
-            emit_dim(b, n0, hv.stride[0], rv.stride[0], oth, hv.io, rv.io, +1, ops);
+            const size_t mark   = plan.passes.size();
+            try
+            {
+                emit_dim(b, n0, hv.stride[0], rv.stride[0], oth, hv.io, rv.io, +1, ops);
+            }
+            catch(const PlanError&)
+            {
+                plan.passes.resize(mark);
+                std::vector<Other> lines; // is = real side, os = Hermitian side
+                for(const Other& o : oth)
+                    lines.push_back({o.cnt, o.os, o.is});
+                emit_odd_real_via_complex(b, false, n0, lines, rv.stride[0], rv.io, hv.stride[0], hv.io,
+                                          p.scale, p.has_scale);
+            }
         }
         return rocfft_status_success;
     }
@@ -1924,6 +2046,7 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
     const size_t scalar = plan.precision ? 8 : 4;
     char*        tmp    = static_cast<char*>(work);
     char*        blu    = tmp ? tmp + plan.tmp_elems * plan.elem_bytes : nullptr;
+    char*        cpx    = tmp ? blu + plan.blu_elems * plan.elem_bytes : nullptr;
     auto resolve = [&](const IoRef& io, char*& p0, char*& p1) -> bool {
         char* base0 = nullptr;
         char* base1 = nullptr;
@@ -1939,6 +2062,9 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             break;
         case BUF_TMP:
             base0 = tmp;
+            break;
+        case BUF_CPX:
+            base0 = cpx;
             break;
         default:
             base0 = blu;
@@ -1971,6 +2097,15 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             if(!aligned(s0, 8) || !aligned(d0, 8))
                 return rocfft_status_failure;
             rc = fftrt_launch_big32k(&q, stream);
+        }
+        else if(rec.kind == PASS_COPY)
+        {
+            fftk_copy_params c = rec.cp;
+            c.s0               = s0;
+            c.s1               = s1;
+            c.d0               = d0;
+            c.d1               = d1;
+            rc                 = fftrt_launch_copy(&c, plan.precision, stream);
         }
         else if(rec.kind == PASS_TILE)
         {
@@ -2030,6 +2165,8 @@ static const char* buf_name(int b)
         return "out";
     case BUF_TMP:
         return "tmp";
+    case BUF_CPX:
+        return "cpx";
     default:
         return "blu";
     }
@@ -2063,6 +2200,8 @@ std::string ExecPlan::describe() const
         }
         else if(r.kind == PASS_BIG)
             o << " threads 1024 grid " << r.grid << " lds 135296";
+        else if(r.kind == PASS_COPY)
+            o << " rows " << r.cp.rows0 << "x" << r.cp.rows1 << "x" << r.cp.rows2;
         else
             o << " half " << r.rp.half << " rows " << r.rp.rows0 << "x" << r.rp.rows1 << "x"
               << r.rp.rows2;

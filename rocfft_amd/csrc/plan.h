@@ -24,7 +24,8 @@ enum BufId
     BUF_IN  = 0, // user input
     BUF_OUT = 1, // user output
     BUF_TMP = 2, // work buffer, general scratch region
-    BUF_BLU = 3  // work buffer, Bluestein region
+    BUF_BLU = 3, // work buffer, Bluestein region
+    BUF_CPX = 4  // work buffer, complex copy of a real transform's rows
 };
 
 // a device-resident table, shared between plans through the table cache
@@ -57,7 +58,8 @@ enum PassKind
     PASS_TILE      = 0,
     PASS_REAL_POST = 1,
     PASS_REAL_PRE  = 2,
-    PASS_BIG       = 3 // one-workgroup 32768-point single-precision kernel
+    PASS_BIG       = 3, // one-workgroup 32768-point single-precision kernel
+    PASS_COPY      = 4  // element-wise row copy between array kinds
 };
 
 // where a pass finds one side of its data: buffer, planar or not, scalar offsets
@@ -76,6 +78,7 @@ struct PassRec
     fftk_params           kp;
     fftk_real_params      rp;
     fftk_big_params       bp;
+    fftk_copy_params      cp;
     IoRef                 src, dst;
     bool                  vec_ok = false;
     bool                  lean_ok = false; // eligible for the branch-free addressing path when vec holds
@@ -92,11 +95,12 @@ struct ExecPlan
     int                  precision  = 0; // 0 float, 1 double
     size_t               tmp_elems  = 0; // complex elements of general scratch
     size_t               blu_elems  = 0; // complex elements of Bluestein scratch
+    size_t               cpx_elems  = 0; // complex elements of the real-as-complex scratch
     size_t               elem_bytes = 8; // bytes per complex element
     bool                 inplace    = false;
     size_t               work_bytes() const
     {
-        return (tmp_elems + blu_elems) * elem_bytes;
+        return (tmp_elems + blu_elems + cpx_elems) * elem_bytes;
     }
     std::string describe() const;
 };

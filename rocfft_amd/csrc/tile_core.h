@@ -582,4 +582,37 @@ FFT_DEV void real_pre_elem(const fftk_real_params& p, uint64_t gid)
     }
 }
 
+// one element of a row copy (fftk_copy_params)
+template <typename T>
+FFT_DEV void copy_elem(const fftk_copy_params& p, uint64_t gid)
+{
+    uint32_t j  = (uint32_t)(gid % p.cnt);
+    uint64_t r  = gid / p.cnt;
+    uint32_t r0 = (uint32_t)(r % p.rows0);
+    r /= p.rows0;
+    uint32_t r1 = (uint32_t)(r % p.rows1);
+    uint32_t r2 = (uint32_t)(r / p.rows1);
+    if(r2 >= p.rows2)
+        return;
+    const int64_t sb   = (int64_t)r0 * p.s_r0 + (int64_t)r1 * p.s_r1 + (int64_t)r2 * p.s_r2;
+    const int64_t db   = (int64_t)r0 * p.d_r0 + (int64_t)r1 * p.d_r1 + (int64_t)r2 * p.d_r2;
+    const bool    flip = p.mirror_from && j >= p.mirror_from;
+    const int64_t so   = sb + (int64_t)(flip ? p.mirror_n - j : j) * p.s_s;
+    T             re   = static_cast<const T*>(p.s0)[so];
+    T             im   = p.src_real ? (T)0 : static_cast<const T*>(p.s1)[so];
+    if(flip)
+        im = -im;
+    if(p.zero_im0 && j == 0)
+        im = 0;
+    if(p.use_scale)
+    {
+        re *= (T)p.scale;
+        im *= (T)p.scale;
+    }
+    const int64_t dof           = db + (int64_t)j * p.d_s;
+    static_cast<T*>(p.d0)[dof] = re;
+    if(!p.dst_real)
+        static_cast<T*>(p.d1)[dof] = im;
+}
+
 #endif

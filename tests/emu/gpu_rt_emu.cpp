@@ -207,6 +207,14 @@ int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void*
     return 0;
 }
 
+int fftrt_launch_copy(const struct fftk_copy_params* p, int precision, void*)
+{
+    uint64_t total = (uint64_t)p->cnt * p->rows0 * p->rows1 * p->rows2;
+    for(uint64_t g = 0; g < total; ++g)
+        precision ? copy_elem<double>(*p, g) : copy_elem<float>(*p, g);
+    return 0;
+}
+
 int fftrt_has_big32k(void)
 {
     return 0;

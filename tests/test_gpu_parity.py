@@ -104,6 +104,15 @@ def test_long_1d(gpu, n):
         H.check(lib, be, B.REAL_INVERSE, [n], 2, B.DOUBLE, inplace=True)
 
 
+@pytest.mark.parametrize("lengths", [[8193], [10007], [19683], [15625], [100003], [9999, 3], [3, 9999]])
+def test_long_odd_real(gpu, lengths):
+    lib, be = gpu
+    H.check(lib, be, B.REAL_FORWARD, lengths, 2, B.DOUBLE)
+    H.check(lib, be, B.REAL_INVERSE, lengths, 2, B.SINGLE)
+    H.check(lib, be, B.REAL_FORWARD, lengths, 2, B.SINGLE, inplace=True, scale=0.25)
+    H.check(lib, be, B.REAL_INVERSE, lengths, 2, B.DOUBLE, inplace=True)
+
+
 @pytest.mark.parametrize("lengths", [[8, 8], [64, 64], [100, 30], [17, 19], [1024, 1024], [4096, 64], [64, 4096],
                                      [8, 8, 8], [16, 8, 4], [30, 20, 10], [128, 32, 8], [5, 7, 9], [8192, 4], [4, 8192], [64, 64, 64],
                                      [128, 128, 128], [512, 16, 16], [16, 512, 4], [8, 4, 512], [1, 8], [8, 1, 4]])

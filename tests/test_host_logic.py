@@ -287,6 +287,20 @@ def test_long_1d(emu, lengths):
         H.check(emu, HOST, B.REAL_INVERSE, lengths, 1, B.DOUBLE, inplace=True)
 
 
+@pytest.mark.parametrize("lengths", [[8193], [10007], [19683], [15625], [9999, 3], [3, 9999]])
+def test_long_odd_real(emu, lengths):
+    """Odd real lengths beyond one kernel go through a complex scratch copy (split or Bluestein
+    in between); the first dimension is the real one."""
+    H.check(emu, HOST, B.REAL_FORWARD, lengths, 2, B.DOUBLE)
+    H.check(emu, HOST, B.REAL_INVERSE, lengths, 2, B.SINGLE)
+    if lengths[0] > 8192:
+        H.check(emu, HOST, B.REAL_FORWARD, lengths, 2, B.SINGLE, inplace=True, scale=0.25)
+        H.check(emu, HOST, B.REAL_INVERSE, lengths, 2, B.DOUBLE, inplace=True)
+        st, text, work = emu.describe(B.NOTINPLACE, B.REAL_FORWARD, B.DOUBLE, lengths, 2)
+        assert st == 0 and "real rows to complex scratch" in text and "first bins to Hermitian rows" in text
+        assert work >= 2 * int(np.prod(lengths)) * 16
+
+
 @pytest.mark.parametrize("lengths", [[8, 8], [64, 64], [100, 30], [30, 100], [17, 19], [1024, 1024], [4, 2048],
                                      [2048, 4], [8, 8, 8], [16, 8, 4], [4, 8, 16], [30, 20, 10], [128, 32, 8],
                                      [5, 7, 9], [8192, 4], [4, 8192], [64, 64, 64], [2, 2, 2], [1, 8], [8, 1, 4]])
