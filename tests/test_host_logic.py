@@ -232,7 +232,7 @@ def test_compiled_schedule_list_is_consistent(emu):
     assert len(rows) == len({r[0] for r in rows}) and len(rows) > 200
     for n, radix, tf, td in rows:
         assert int(np.prod(radix)) == n and 1 <= len(radix) <= 4
-        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 16) for r in radix)
+        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13, 16) for r in radix)
         need = max(-(-(n // r) // (16 // r)) for r in radix)
         for t in (tf, td):
             assert t == 0 or need <= t <= 512
