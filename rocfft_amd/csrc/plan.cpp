@@ -1163,20 +1163,49 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         if(n1 == 0)
             fail("length too large for the two- and three-pass decompositions");
         // pass A: for every n0' an n1-point FFT over the stride-n0 samples, times W_n^{k1 n0'},
-        // written to scratch at [line][k1*n0 + n0']
+        // written to scratch at index k1*n0 + n0' of the dimension
         // pass B: for every k1 an n0-point FFT over n0', written to dst at k0*n1 + k1
         // (the reference's two-kernel large 1D, library/src/tree_node_1D.cpp:404-469)
-        b.need_tmp(lines * n);
-        std::vector<int64_t> pk = packed_strides(n);
-        TablePtr             ltw = large_twiddles(n, b.precision, b.dry);
+        //
+        // The scratch array keeps the axis order of the source: axes that run faster than this
+        // dimension in the source (the columns of a strided dimension) stay innermost, so that
+        // a tile of neighbouring columns is contiguous in the scratch array too; the other axes
+        // are packed outside the dimension.
+        std::vector<int64_t> pk(others.size(), 0);
+        std::vector<size_t>  order(others.size());
+        for(size_t i = 0; i < others.size(); ++i)
+            order[i] = i;
+        std::sort(order.begin(), order.end(),
+                  [&](size_t x, size_t y) { return others[x].is < others[y].is; });
+        int64_t inner = 1; // complex elements inside one step of this dimension
+        for(size_t i : order)
+            if(others[i].cnt > 1 && others[i].is < t_is)
+            {
+                pk[i] = 2 * inner;
+                inner *= others[i].cnt;
+            }
+        // keep the pitch of the dimension off multiples of 2 KiB (HBM channel aliasing)
+        int64_t innerP = inner;
+        if(inner > 1 && ((size_t)inner * esize) % 2048 == 0)
+            innerP += 16;
+        const int64_t tS    = 2 * innerP; // scalar stride of the dimension in the scratch array
+        int64_t       outer = (int64_t)n * tS;
+        for(size_t i : order)
+            if(!(others[i].cnt > 1 && others[i].is < t_is))
+            {
+                pk[i] = outer;
+                outer *= others[i].cnt;
+            }
+        b.need_tmp((size_t)(outer / 2));
+        TablePtr ltw = large_twiddles(n, b.precision, b.dry);
         {
             TileSpec s = base_spec();
             s.n        = (uint32_t)n1;
             s.t_is     = (int64_t)n0 * t_is;
-            s.t_os     = (int64_t)n0 * 2;
+            s.t_os     = (int64_t)n0 * tS;
             s.src      = src;
             s.dst      = tmp;
-            s.others.push_back({(uint32_t)n0, t_is, 2, true});
+            s.others.push_back({(uint32_t)n0, t_is, tS, true});
             add_others(s, true, false, pk);
             s.flags |= FFTK_F_TWIDDLE_STORE;
             s.ltw       = ltw;
@@ -1187,18 +1216,18 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         {
             TileSpec s = base_spec();
             s.n        = (uint32_t)n0;
-            s.t_is     = 2;
+            s.t_is     = tS;
             s.t_os     = (int64_t)n1 * t_os;
             s.src      = tmp;
             s.dst      = dst;
-            s.others.push_back({(uint32_t)n1, (int64_t)n0 * 2, t_os, false});
+            s.others.push_back({(uint32_t)n1, (int64_t)n0 * tS, t_os, false});
             add_others(s, false, true, pk);
             if(ops.has_scale)
             {
                 s.flags |= FFTK_F_SCALE;
                 s.scale = ops.scale;
             }
-            s.note = dims_note("split B (row fft, transposed store)", n0);
+            s.note = dims_note(inner > 1 ? "split B (column fft, transposed store)" : "split B (row fft, transposed store)", n0);
             b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
         }
         return;
