@@ -24,10 +24,11 @@ namespace
 // 2: the lean path (vector accesses, interleaved complex on both sides)
 // Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
 // their tile rows wide); no kernel here needs more than the 256 registers that leaves a thread.
+// The longest lengths need up to 1024 threads for one transform (128 registers a thread).
 template <typename Cfg>
 constexpr int fast_block_limit()
 {
-    return 512;
+    return Cfg::TPT > 512 ? 1024 : 512;
 }
 
 template <typename T, typename Cfg, int MODE>
@@ -66,8 +67,10 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* str
 #define FAST_ONE_0(T, P, N, A, B, C, D, TT)                                                            \
     {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
      nullptr, nullptr},
-#define FAST_ENTRY(FULL, N, A, B, C, D, TTF, TTD) \
-    FAST_ONE_##FULL(float, 0, N, A, B, C, D, TTF) FAST_ONE_##FULL(double, 1, N, A, B, C, D, TTD)
+#define FAST_DBL_1(FULL, N, A, B, C, D, TTD) FAST_ONE_##FULL(double, 1, N, A, B, C, D, TTD)
+#define FAST_DBL_0(FULL, N, A, B, C, D, TTD)
+#define FAST_ENTRY(FULL, N, A, B, C, D, TTF, TTD, DBL) \
+    FAST_ONE_##FULL(float, 0, N, A, B, C, D, TTF) FAST_DBL_##DBL(FULL, N, A, B, C, D, TTD)
 
 #define FAST_PICK_0(...)
 #define FAST_PICK_1(...)
@@ -204,7 +207,7 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
                                       size_t lds_bytes, void* stream)
 {
     const FastEntry* e = find_fast(precision, p->n);
-    if(!e || p->T != e->tpt || p->nthreads > 512u || p->padshift != 4)
+    if(!e || p->T != e->tpt || p->nthreads > (e->tpt > 512 ? 1024u : 512u) || p->padshift != 4)
         return (int)hipErrorInvalidValue;
     uint32_t cnt = 0;
     for(uint32_t i = 0; i < 4; ++i)

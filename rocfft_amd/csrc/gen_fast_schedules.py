@@ -15,6 +15,12 @@ import sys
 REG_ELEMS = 16
 RADICES = [16, 13, 11, 10, 9, 8, 7, 6, 5, 4, 3, 2]
 MAX_N = 4096
+# Longer lengths (prime factors up to 5) that one workgroup of up to 1024 threads transforms
+# in LDS in single precision; double precision where 512 threads and 160 KB of LDS suffice.
+WIDE_LENGTHS = [4320, 4374, 4500, 4608, 4800, 4860, 5000, 5120, 5184, 5400, 5760, 5832, 6000, 6144, 6400,
+                6480, 6561, 6912, 7200, 7290, 7680, 7776, 8000, 8100, 8640, 9000, 9216, 9600, 10000, 10240,
+                12288, 16384]
+LDS_BYTES = 160 * 1024
 SLICES = 8
 
 # Threads per transform (single, double precision) where the default -- the fewest the
@@ -145,7 +151,12 @@ def lane_work(n, sched):
     return t * sum(((n // r + t - 1) // t) * r for r in sched)
 
 
-def best_schedule(n):
+def lds_bytes(n, elem_bytes):
+    pitch = (n + ((n - 1) >> 4) + 1) | 1
+    return pitch * elem_bytes
+
+
+def best_schedule(n, max_threads=512):
     best = None
     for npass in range(1, 5):
         for combo in itertools.combinations_with_replacement(RADICES, npass):
@@ -155,7 +166,7 @@ def best_schedule(n):
             if prod != n:
                 continue
             t = tpt(n, combo)
-            if t > 512:
+            if t > max_threads:
                 continue
             # fewer passes first, then the least lane work, then the larger radices
             key = (npass, lane_work(n, combo), tuple(-r for r in combo))
@@ -231,11 +242,14 @@ def main():
         s = TUNED_SCHEDULE.get(n) or best_schedule(n)
         if s:
             rows.append((n, s, 0))
+    for n in WIDE_LENGTHS:
+        s = TUNED_SCHEDULE.get(n) or best_schedule(n, 1024)
+        rows.append((n, s, 0))
     out = sys.stdout
     out.write("// fast_schedules.h -- generated by gen_fast_schedules.py, do not edit.\n")
-    out.write("// FAST_SCHED(slice, all_modes, N, R0, R1, R2, R3, TPTF, TPTD): length N runs the passes R0..R3\n")
+    out.write("// FAST_SCHED(slice, all_modes, N, R0, R1, R2, R3, TPTF, TPTD, DBL): length N runs the passes R0..R3\n")
     out.write("// (1 = unused) with TPTF / TPTD threads per transform in single / double precision (0 = the\n")
-    out.write("// fewest the register budget allows);\n")
+    out.write("// fewest the register budget allows); DBL = 0: no double-precision kernel (it would not fit);\n")
     out.write("// all_modes = 1 builds the scalar and general vector variants besides the lean one;\n")
     out.write("// slice names the translation unit that instantiates the kernels.\n")
     out.write("#define FAST_SLICES %d\n" % SLICES)
@@ -255,8 +269,9 @@ def main():
             variants = [(s, tf, td)]
         for sc, tf, td in variants:
             r = list(sc) + [1] * (4 - len(sc))
-            out.write("FAST_SCHED(%d, %d, %d, %d, %d, %d, %d, %d, %d)\n"
-                      % (slice_of[n], full, n, r[0], r[1], r[2], r[3], tf, td))
+            dbl = 1 if (max(td, tpt(n, sc)) <= 512 and lds_bytes(n, 16) <= LDS_BYTES) else 0
+            out.write("FAST_SCHED(%d, %d, %d, %d, %d, %d, %d, %d, %d, %d)\n"
+                      % (slice_of[n], full, n, r[0], r[1], r[2], r[3], tf, td, dbl))
     sys.stderr.write("%d lengths\n" % len(rows))
 
 

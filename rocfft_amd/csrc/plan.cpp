@@ -23,6 +23,8 @@ static const size_t   LDS_HARD_BYTES = 160 * 1024; // LDS of one CU
 static const size_t   LDS_COL_BYTES  = 80 * 1024;  // a column tile may grow to this to keep its rows wide
 static const size_t   LDS_WIDE_BYTES = 140 * 1024; // ... and to this when the alternative is a second pass
 static const uint32_t MAX_THREADS    = 512;
+// a few compiled kernels for long single-precision rows use one workgroup of up to this many threads
+static const uint32_t WIDE_THREADS   = 1024;
 static const uint32_t PADSHIFT       = 4;
 // a strided ("column") pass wants at least this many bytes contiguous per row of its tile
 static const size_t   COL_RUN_BYTES  = 128;
@@ -372,6 +374,19 @@ static bool single_kernel_length(uint64_t n, size_t elem_bytes)
     return (size_t)lds_pitch((uint32_t)n) * elem_bytes <= LDS_HARD_BYTES;
 }
 
+// Lengths that only a compiled kernel with more than MAX_THREADS threads per transform can
+// take in one pass (no generic-kernel fallback exists for them: the pass must be able to use
+// the kernel's lean variant).
+static bool wide_kernel_length(uint64_t n, size_t elem_bytes)
+{
+    std::vector<uint32_t> radix;
+    bool                  fast = false;
+    uint32_t              T    = kernel_schedule(n, elem_bytes == 16 ? 1 : 0, radix, &fast);
+    if(!fast || T <= MAX_THREADS || T > WIDE_THREADS)
+        return false;
+    return (size_t)lds_pitch((uint32_t)n) * elem_bytes <= LDS_HARD_BYTES;
+}
+
 // longest length a strided pass handles while keeping COL_RUN_BYTES contiguous per row
 static bool column_kernel_length(uint64_t n, size_t elem_bytes)
 {
@@ -646,7 +661,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     k.T        = sched_T;
     k.padshift = PADSHIFT;
     k.pitch    = lds_pitch(s.n);
-    if(k.T > MAX_THREADS)
+    if(k.T > MAX_THREADS && !(have_fast && k.T <= WIDE_THREADS))
         fail("transform too long for one workgroup");
     // a kernel compiled for exactly this pass schedule, when there is one
     uint32_t max_threads = MAX_THREADS;
@@ -656,7 +671,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         k.fast      = 1;
         k.T         = fast_tpt;
         // a strided pass may use the larger workgroup to keep its tile rows wide
-        max_threads = (fast_tpt > 256 || k.in_fast_tile || k.out_fast_tile) ? 512 : 256;
+        max_threads = fast_tpt > 512 ? WIDE_THREADS
+                                     : (fast_tpt > 256 || k.in_fast_tile || k.out_fast_tile) ? 512 : 256;
     }
     size_t   per_tile  = (size_t)k.pitch * esize;
     uint32_t w_threads = floor_pow2(max_threads / k.T);
@@ -788,6 +804,9 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             }
         }
     }
+
+    if(k.T > MAX_THREADS && !rec.lean_ok)
+        fail("no kernel for a transform this long in this layout");
 
     // data volume of the pass: every element it loads plus every element it stores
     {
@@ -1062,8 +1081,7 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
 
     // a pass that is not "plain" (fused real/odd handling) stays single if it fits at all
     bool single = plain ? plain_dim_is_single(n, column, esize, t_is, t_os) : single_kernel_length(n, esize);
-    if(single)
-    {
+    auto emit_single = [&]() {
         TileSpec s = base_spec();
         s.n        = (uint32_t)n;
         s.t_is     = t_is;
@@ -1085,7 +1103,25 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         }
         s.note = dims_note(column ? "column fft" : "row fft", n);
         b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    };
+    if(single)
+    {
+        emit_single();
         return;
+    }
+    // one workgroup of up to 1024 threads, when the layout suits the compiled kernel's lean variant
+    if(!column && wide_kernel_length(n, esize))
+    {
+        const size_t mark = b.plan->passes.size();
+        try
+        {
+            emit_single();
+            return;
+        }
+        catch(const PlanError&)
+        {
+            b.plan->passes.resize(mark);
+        }
     }
 
     if(smooth(n))
@@ -1831,6 +1867,33 @@ static std::vector<Other> other_axes(const View& in, const View& out, const size
     return o;
 }
 
+// Even-length real transform whose half length needs a wide kernel: the fused variant, if the
+// layout allows it.  Leaves the pass list untouched and returns false otherwise.
+static bool try_fused_real(Builder& b, bool forward, uint64_t half, int64_t t_is, int64_t t_os,
+                           const std::vector<Other>& oth, const IoRef& src, const IoRef& dst, double scale,
+                           bool has_scale)
+{
+    DimOps ops;
+    if(forward)
+        ops.store_op = FFTK_STORE_R2C_POST;
+    else
+        ops.load_op = FFTK_LOAD_C2R_PRE;
+    ops.half_tw   = half_twiddles(half, b.precision, b.dry);
+    ops.scale     = scale;
+    ops.has_scale = has_scale;
+    const size_t mark = b.plan->passes.size();
+    try
+    {
+        emit_dim(b, half, t_is, t_os, oth, src, dst, forward ? -1 : +1, ops);
+        return true;
+    }
+    catch(const PlanError&)
+    {
+        b.plan->passes.resize(mark);
+        return false;
+    }
+}
+
 static void check_sizes(const Problem& p)
 {
     for(size_t d = 0; d < p.rank; ++d)
@@ -1916,6 +1979,12 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                     }
                     emit_dim(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, -1, ops);
                 }
+                else if(wide_kernel_length(half, b.esize)
+                        && try_fused_real(b, true, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io, p.scale,
+                                          last0 && p.has_scale))
+                {
+                    // one wide kernel with the post-processing fused
+                }
                 else
                 {
                     // half-length complex FFT into the output rows, then the
@@ -1985,6 +2054,12 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                 ops.scale     = p.scale;
                 ops.has_scale = p.has_scale;
                 emit_dim(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io, +1, ops);
+            }
+            else if(wide_kernel_length(half, b.esize)
+                    && try_fused_real(b, false, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io, p.scale,
+                                      p.has_scale))
+            {
+                // one wide kernel with the pre-processing fused
             }
             else
             {

@@ -154,8 +154,8 @@ struct EmuSched
 {
     uint32_t n, radix[4], tpt[2]; // threads per transform in single, double precision
 };
-#define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD) \
-    {N, {A, B, C, D}, {(uint32_t)FastCfg<N, A, B, C, D, TTF>::TPT, (uint32_t)FastCfg<N, A, B, C, D, TTD>::TPT}},
+#define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD, DBL) \
+    {N, {A, B, C, D}, {(uint32_t)FastCfg<N, A, B, C, D, TTF>::TPT, (DBL) ? (uint32_t)FastCfg<N, A, B, C, D, TTD>::TPT : 0u}},
 const EmuSched g_sched[] = {
 #include "fast_schedules.h"
 };
@@ -181,7 +181,7 @@ uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* radix, uint32_
 int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
                       size_t lds_bytes, void*)
 {
-    if(p->nthreads == 0 || p->nthreads > 512 || (p->nthreads & 63) || lds_bytes > 160 * 1024
+    if(p->nthreads == 0 || p->nthreads > 1024 || (p->nthreads & 63) || lds_bytes > 160 * 1024
        || grid == 0)
         return 1;
     if(precision == 0)

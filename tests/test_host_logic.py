@@ -235,7 +235,7 @@ def test_compiled_schedule_list_is_consistent(emu):
         assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13, 16) for r in radix)
         need = max(-(-(n // r) // (16 // r)) for r in radix)
         for t in (tf, td):
-            assert t == 0 or need <= t <= 512
+            assert t == 0 or need <= t <= 1024
     for n, radix, tf, td in rows[::7]:
         st, text, _ = emu.describe(B.NOTINPLACE, 0, 0, [n], 4)
         assert st == 0
