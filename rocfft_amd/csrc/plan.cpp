@@ -1285,16 +1285,17 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     bool one = column ? column_kernel_length(M, esize) : single_kernel_length(M, esize);
     if(!one && column && single_kernel_length(M, esize) && M <= 4096)
         one = true;
+    // single precision: M = 16384 still fits one workgroup of the wide compiled kernel
+    const bool wide_one = !one && !column && wide_kernel_length(M, esize);
     // (checked before any table is computed: a chirp of 10^8 entries takes a minute)
-    if(!one && (ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out))
+    if(!one && !wide_one && (ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out))
         fail("odd-length real transforms of this size are not implemented");
     if(!one && !single_kernel_length(M / 4096, esize))
         fail("Bluestein length too large");
     TablePtr chirp      = chirp_table(N, b.precision, b.dry);
     double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
     uint32_t cflag      = conj_chirp ? FFTK_F_CHIRP_CONJ : 0;
-    if(one)
-    {
+    auto emit_one = [&]() {
         TablePtr bs = bluestein_spectrum(b, N, M, 0, 0, conj_chirp);
         TileSpec s  = base_spec();
         s.dir       = -1;
@@ -1320,7 +1321,24 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         s.scale    = scale;
         s.note     = dims_note("bluestein single kernel, M", M);
         b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+    };
+    if(one)
+    {
+        emit_one();
         return;
+    }
+    if(wide_one)
+    {
+        const size_t mark = b.plan->passes.size();
+        try
+        {
+            emit_one();
+            return;
+        }
+        catch(const PlanError&)
+        {
+            b.plan->passes.resize(mark);
+        }
     }
     if(ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out)
         fail("odd-length real transforms of this size are not implemented");
@@ -1477,7 +1495,14 @@ static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t 
             sub.passes.push_back(make_tile_pass(r, 1, false));
         }
         void* bufs[2] = {dbuf, nullptr};
-        if(run_exec_plan(sub, bufs, bufs, nullptr, nullptr) != rocfft_status_success)
+        void* sub_work = nullptr;
+        if(sub.work_bytes() && fftrt_malloc(&sub_work, sub.work_bytes()) != 0)
+            fail("device allocation failed");
+        std::shared_ptr<void> work_guard(sub_work, [](void* p) {
+            if(p)
+                fftrt_free(p);
+        });
+        if(run_exec_plan(sub, bufs, bufs, sub_work, nullptr) != rocfft_status_success)
             fail("computing the Bluestein chirp spectrum failed");
         if(fftrt_stream_sync(nullptr) != 0)
             fail("computing the Bluestein chirp spectrum failed");
