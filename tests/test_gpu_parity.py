@@ -182,11 +182,11 @@ def test_c2r_ignores_imaginary_dc_and_nyquist(gpu):
 def test_work_buffer_contract(gpu):
     lib, be = gpu
     torch = be.torch
-    n = 8191
-    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], 1, lib=lib)
+    n = 8191  # double precision: three Bluestein kernels and a work buffer
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.DOUBLE, [n], 1, lib=lib)
     need = plan.work_buffer_size
     assert need > 0
-    x = torch.zeros(n, dtype=torch.complex64, device=be.dev)
+    x = torch.zeros(n, dtype=torch.complex128, device=be.dev)
     x[1] = 1
     y = torch.zeros_like(x)
     plan.execute([x.data_ptr()], [y.data_ptr()])  # scratch allocated by execute

@@ -143,11 +143,11 @@ def test_distributed_descriptions_are_rejected(emu):
 def test_work_buffer_contract(emu):
     # reference clients/tests/unit_test.cpp:256-345 (N=8191, Bluestein): missing buffer is
     # allocated by execute, a short one is rejected at execute
-    n = 8191
-    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], 1, lib=emu)
+    n = 8191  # double precision: three Bluestein kernels and a work buffer
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.DOUBLE, [n], 1, lib=emu)
     need = plan.work_buffer_size
     assert need > 0
-    x = np.zeros(n, dtype=np.complex64)
+    x = np.zeros(n, dtype=np.complex128)
     x[1] = 1
     y = np.zeros_like(x)
     plan.execute([x.ctypes.data], [y.ctypes.data])  # auto-allocated
