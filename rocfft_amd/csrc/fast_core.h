@@ -385,30 +385,55 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     {
         // r holds the forward spectrum: multiply by the stored spectrum, exchange re/im and
         // run the passes again, which makes the second transform an inverse one
-        if(Cfg::NP > 1 || lds_busy)
-            __syncthreads();
-        if(active)
+        const C* cb = static_cast<const C*>(p.convb) + (uint64_t)q * p.convb_qs;
+        if constexpr(RL == R0)
         {
-            const C* cb = static_cast<const C*>(p.convb) + (uint64_t)q * p.convb_qs;
+            // equal first and last radix: the last pass leaves a thread exactly the elements
+            // its first pass takes (tt + s TPT + k N/R), so the spectrum stays in registers
+            if(active)
+            {
 #pragma unroll
-            for(int s = 0; s < SL; ++s)
+                for(int s = 0; s < SL; ++s)
 #pragma unroll
-                for(int k = 0; k < RL; ++k)
-                {
-                    const uint32_t j = tt + s * Cfg::TPT + k * CL;
-                    if(!fk_live<Cfg, LAST>(tt, s))
-                        continue;
-                    C v = r[s * RL + k];
-                    if(ok)
-                        v = c_mul(v, cb[j]);
-                    lds[fk_addr<Cfg>(w, j)] = c_swap(v);
-                }
+                    for(int k = 0; k < RL; ++k)
+                    {
+                        const uint32_t j = tt + s * Cfg::TPT + k * CL;
+                        if(!fk_live<Cfg, LAST>(tt, s))
+                            continue;
+                        C v = r[s * RL + k];
+                        if(ok)
+                            v = c_mul(v, cb[j]);
+                        r[s * RL + k] = c_swap(v);
+                    }
+            }
+            fk_passes<T, Cfg>(p, lds, w, tt, active, r, Cfg::NP > 1 || lds_busy);
         }
-        __syncthreads();
-        if(active)
-            fk_read<T, Cfg, 0>(lds, w, tt, r);
-        fk_passes<T, Cfg>(p, lds, w, tt, active, r, true);
-        lds_busy = true;
+        else
+        {
+            if(Cfg::NP > 1 || lds_busy)
+                __syncthreads();
+            if(active)
+            {
+#pragma unroll
+                for(int s = 0; s < SL; ++s)
+#pragma unroll
+                    for(int k = 0; k < RL; ++k)
+                    {
+                        const uint32_t j = tt + s * Cfg::TPT + k * CL;
+                        if(!fk_live<Cfg, LAST>(tt, s))
+                            continue;
+                        C v = r[s * RL + k];
+                        if(ok)
+                            v = c_mul(v, cb[j]);
+                        lds[fk_addr<Cfg>(w, j)] = c_swap(v);
+                    }
+            }
+            __syncthreads();
+            if(active)
+                fk_read<T, Cfg, 0>(lds, w, tt, r);
+            fk_passes<T, Cfg>(p, lds, w, tt, active, r, true);
+        }
+        lds_busy = lds_busy || Cfg::NP > 1 || RL != R0;
         out_inv  = true;
     }
 
