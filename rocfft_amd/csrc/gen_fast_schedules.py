@@ -71,6 +71,7 @@ TUNED_TPT = {
 }
 # pass schedules where the default (fewest passes, least lane work) is not the fastest
 TUNED_SCHEDULE = {
+    16384: (16, 16, 4, 16),
     12: (4, 3), 15: (3, 5), 18: (6, 3), 20: (5, 4), 24: (4, 6), 30: (6, 5), 35: (5, 7),
     40: (4, 10), 42: (6, 7), 48: (8, 6), 55: (5, 11), 56: (7, 8), 63: (7, 9), 70: (7, 10),
     72: (8, 9), 77: (7, 11), 78: (6, 13), 80: (5, 16), 88: (8, 11), 90: (9, 10), 96: (6, 16),
