@@ -216,6 +216,25 @@ class ExecutionInfo:
         self.lib.check(st, "rocfft_execution_info_set_stream")
         return self
 
+    def _set_callback(self, name, fn, data, shared_mem_bytes):
+        fns = (ctypes.c_void_p * 1)(fn)
+        datas = (ctypes.c_void_p * 1)(data)
+        return getattr(self.lib.c, name)(self.handle, fns, datas, shared_mem_bytes)
+
+    def set_load_callback(self, fn, data=None, shared_mem_bytes=0):
+        """fn: device address of `T load_cb(T* data, size_t offset, void* cbdata, void* sharedMem)`
+        (None clears it); data: the cbdata pointer"""
+        st = self._set_callback("rocfft_execution_info_set_load_callback", fn, data, shared_mem_bytes)
+        self.lib.check(st, "rocfft_execution_info_set_load_callback")
+        return self
+
+    def set_store_callback(self, fn, data=None, shared_mem_bytes=0):
+        """fn: device address of `void store_cb(T* data, size_t offset, T element, void* cbdata,
+        void* sharedMem)` (None clears it)"""
+        st = self._set_callback("rocfft_execution_info_set_store_callback", fn, data, shared_mem_bytes)
+        self.lib.check(st, "rocfft_execution_info_set_store_callback")
+        return self
+
     def destroy(self):
         if self.handle:
             self.lib.c.rocfft_execution_info_destroy(self.handle)

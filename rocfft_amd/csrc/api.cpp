@@ -48,6 +48,10 @@ struct rocfft_execution_info_t
     void*  workBuffer     = nullptr;
     size_t workBufferSize = 0;
     void*  stream         = nullptr;
+    void*  load_cb        = nullptr; // device address of the load callback, its data
+    void*  load_cb_data   = nullptr;
+    void*  store_cb       = nullptr;
+    void*  store_cb_data  = nullptr;
 };
 
 struct rocfft_field_t
@@ -481,12 +485,100 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         }
         if(pass_ms && fftrt_stream_capturing(stream))
             return rocfft_status_failure;
-        rocfft_status st = run_exec_plan(ep, in, out, work, stream, pass_ms);
-        if(own)
+
+        // Load/store callbacks: the input is copied into a scratch buffer of the same layout
+        // through the load callback, the plan runs on scratch buffers, and the result goes to
+        // the user's buffer through the store callback (two extra element-wise passes; the
+        // transform kernels themselves make no indirect calls).
+        void*      cb_in    = nullptr;
+        void*      cb_out   = nullptr;
+        const bool have_cb  = info && (info->load_cb || info->store_cb);
+        auto       cleanup  = [&]() {
+            if(own || cb_in || cb_out)
+                fftrt_stream_sync(stream);
+            if(own)
+                fftrt_free(work);
+            if(cb_in)
+                fftrt_free(cb_in);
+            if(cb_out && cb_out != cb_in)
+                fftrt_free(cb_out);
+        };
+        fftk_cb_params cin, cout;
+        memset(&cin, 0, sizeof(cin));
+        memset(&cout, 0, sizeof(cout));
+        bool in_complex = true, out_complex = true;
+        if(have_cb)
         {
-            fftrt_stream_sync(stream);
-            fftrt_free(work);
+            if(planar(pr.in_type) || planar(pr.out_type) || fftrt_stream_capturing(stream))
+            {
+                cleanup();
+                return rocfft_status_failure;
+            }
+            in_complex  = pr.in_type != rocfft_array_type_real;
+            out_complex = pr.out_type != rocfft_array_type_real;
+            const size_t scalar = pr.precision == rocfft_precision_double ? 8 : 4;
+            auto         fill   = [&](fftk_cb_params& c, bool input) {
+                size_t extent = (input ? pr.ioffset[0] : pr.ooffset[0]) + 1;
+                for(size_t d = 0; d < 3; ++d)
+                {
+                    size_t n = d < pr.rank ? pr.len[d] : 1;
+                    if(d == 0 && ((input && pr.type == rocfft_transform_type_real_inverse)
+                                  || (!input && pr.type == rocfft_transform_type_real_forward)))
+                        n = n / 2 + 1;
+                    c.len[d]    = (uint32_t)n;
+                    c.stride[d] = d < pr.rank ? (int64_t)(input ? pr.istride[d] : pr.ostride[d]) : 0;
+                    extent += (n - 1) * (size_t)c.stride[d];
+                }
+                c.batch  = (uint32_t)pr.batch;
+                c.dist   = (int64_t)(input ? pr.idist : pr.odist);
+                c.offset = (int64_t)(input ? pr.ioffset[0] : pr.ooffset[0]);
+                extent += (pr.batch - 1) * (size_t)c.dist;
+                return extent * scalar * ((input ? in_complex : out_complex) ? 2 : 1);
+            };
+            const size_t in_bytes  = fill(cin, true);
+            const size_t out_bytes = fill(cout, false);
+            const bool   stage_in  = ep.inplace || info->load_cb;
+            const bool   stage_out = ep.inplace || info->store_cb;
+            if(stage_in && fftrt_malloc(&cb_in, ep.inplace ? std::max(in_bytes, out_bytes) : in_bytes) != 0)
+            {
+                cleanup();
+                return rocfft_status_failure;
+            }
+            if(ep.inplace)
+                cb_out = cb_in;
+            else if(stage_out && fftrt_malloc(&cb_out, out_bytes) != 0)
+            {
+                cleanup();
+                return rocfft_status_failure;
+            }
+            if(stage_in)
+            {
+                cin.store   = 0;
+                cin.user    = in[0];
+                cin.scratch = cb_in;
+                cin.fn      = info->load_cb;
+                cin.data    = info->load_cb_data;
+                if(fftrt_launch_callback_copy(&cin, ep.precision, in_complex ? 1 : 0, stream) != 0)
+                {
+                    cleanup();
+                    return rocfft_status_failure;
+                }
+            }
         }
+        void* run_in[2]  = {cb_in ? cb_in : in[0], in[1]};
+        void* run_out[2] = {cb_out ? cb_out : out[0], out[1]};
+        rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms);
+        if(st == rocfft_status_success && cb_out)
+        {
+            cout.store   = 1;
+            cout.user    = out[0];
+            cout.scratch = cb_out;
+            cout.fn      = info->store_cb;
+            cout.data    = info->store_cb_data;
+            if(fftrt_launch_callback_copy(&cout, ep.precision, out_complex ? 1 : 0, stream) != 0)
+                st = rocfft_status_failure;
+        }
+        cleanup();
         return st;
     }
     catch(...)
@@ -779,27 +871,24 @@ rocfft_status rocfft_execution_info_set_stream(rocfft_execution_info info, void*
 rocfft_status rocfft_execution_info_set_load_callback(rocfft_execution_info info, void** cb_functions,
                                                       void** cb_data, size_t shared_mem_bytes)
 {
-    (void)cb_data;
     if(!info)
         return rocfft_status_failure;
     if(shared_mem_bytes)
         return rocfft_status_invalid_arg_value;
-    // clearing a callback is a no-op; installing one needs run-time compiled kernels
-    if(!cb_functions || !cb_functions[0])
-        return rocfft_status_success;
-    return rocfft_status_failure;
+    info->load_cb      = cb_functions ? cb_functions[0] : nullptr;
+    info->load_cb_data = (info->load_cb && cb_data) ? cb_data[0] : nullptr;
+    return rocfft_status_success;
 }
 rocfft_status rocfft_execution_info_set_store_callback(rocfft_execution_info info, void** cb_functions,
                                                        void** cb_data, size_t shared_mem_bytes)
 {
-    (void)cb_data;
     if(!info)
         return rocfft_status_failure;
     if(shared_mem_bytes)
         return rocfft_status_invalid_arg_value;
-    if(!cb_functions || !cb_functions[0])
-        return rocfft_status_success;
-    return rocfft_status_failure;
+    info->store_cb      = cb_functions ? cb_functions[0] : nullptr;
+    info->store_cb_data = (info->store_cb && cb_data) ? cb_data[0] : nullptr;
+    return rocfft_status_success;
 }
 
 rocfft_status rocfft_cache_serialize(void** buffer, size_t* buffer_len_bytes)

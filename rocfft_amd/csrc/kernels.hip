@@ -78,6 +78,12 @@ __global__ __launch_bounds__(256) void real_post_kernel(const fftk_real_params p
     real_post_elem<T>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
 }
 
+template <typename E>
+__global__ __launch_bounds__(256) void callback_copy_kernel(const fftk_cb_params p)
+{
+    callback_elem<E>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void row_copy_kernel(const fftk_copy_params p)
 {
@@ -232,6 +238,25 @@ int fftrt_launch_real_post(const struct fftk_real_params* p, int precision, void
         hipLaunchKernelGGL(real_post_kernel<float>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
     else
         hipLaunchKernelGGL(real_post_kernel<double>, dim3(grid), dim3(256), 0, (hipStream_t)stream, *p);
+    return (int)hipGetLastError();
+}
+
+int fftrt_launch_callback_copy(const struct fftk_cb_params* p, int precision, int complex_elems, void* stream)
+{
+    uint64_t total = (uint64_t)p->len[0] * p->len[1] * p->len[2] * p->batch;
+    uint64_t grid  = (total + 255) / 256;
+    if(grid == 0 || grid >= (1ull << 31))
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = (hipStream_t)stream;
+    dim3        g((uint32_t)grid), b(256);
+    if(precision == 0 && complex_elems)
+        hipLaunchKernelGGL(callback_copy_kernel<float2>, g, b, 0, s, *p);
+    else if(precision == 0)
+        hipLaunchKernelGGL(callback_copy_kernel<float>, g, b, 0, s, *p);
+    else if(complex_elems)
+        hipLaunchKernelGGL(callback_copy_kernel<double2>, g, b, 0, s, *p);
+    else
+        hipLaunchKernelGGL(callback_copy_kernel<double>, g, b, 0, s, *p);
     return (int)hipGetLastError();
 }
 

@@ -141,6 +141,26 @@ struct fftk_copy_params
     uint32_t    use_scale;
 };
 
+// Copy of every element of a transform's input (or output) between the user's buffer and a
+// scratch buffer with the same layout, through the user's load (or store) callback:
+//   T load_cb(T* data, size_t offset, void* cbdata, void* sharedMem);
+//   void store_cb(T* data, size_t offset, T element, void* cbdata, void* sharedMem);
+// (reference library/include/rocfft/rocfft.h:533-612).  Offsets are in elements of the array
+// type (real scalars or complex pairs) from the buffer pointer given to rocfft_execute.
+struct fftk_cb_params
+{
+    uint32_t len[3];
+    uint32_t batch;
+    int64_t  stride[3];
+    int64_t  dist;
+    int64_t  offset;
+    uint32_t store; // 0: user -> scratch through the load callback, 1: scratch -> user through the store callback
+    void*    user;
+    void*    scratch;
+    void*    fn;   // device address of the callback; null = plain copy
+    void*    data; // cbdata
+};
+
 // one-workgroup 32768-point single-precision transform (big_kernels.hip)
 struct fftk_big_params
 {

@@ -582,6 +582,32 @@ FFT_DEV void real_pre_elem(const fftk_real_params& p, uint64_t gid)
     }
 }
 
+// one element of a callback copy (fftk_cb_params); E is the element type of the array
+template <typename E>
+FFT_DEV void callback_elem(const fftk_cb_params& p, uint64_t gid)
+{
+    typedef E (*load_fn)(E*, size_t, void*, void*);
+    typedef void (*store_fn)(E*, size_t, E, void*, void*);
+    uint32_t i0 = (uint32_t)(gid % p.len[0]);
+    gid /= p.len[0];
+    uint32_t i1 = (uint32_t)(gid % p.len[1]);
+    gid /= p.len[1];
+    uint32_t i2 = (uint32_t)(gid % p.len[2]);
+    uint64_t b  = gid / p.len[2];
+    if(b >= p.batch)
+        return;
+    const size_t off = (size_t)(p.offset + (int64_t)b * p.dist + (int64_t)i0 * p.stride[0]
+                                + (int64_t)i1 * p.stride[1] + (int64_t)i2 * p.stride[2]);
+    E* user = static_cast<E*>(p.user);
+    E* scr  = static_cast<E*>(p.scratch);
+    if(!p.store)
+        scr[off] = p.fn ? reinterpret_cast<load_fn>(p.fn)(user, off, p.data, nullptr) : user[off];
+    else if(p.fn)
+        reinterpret_cast<store_fn>(p.fn)(user, off, scr[off], p.data, nullptr);
+    else
+        user[off] = scr[off];
+}
+
 // one element of a row copy (fftk_copy_params)
 template <typename T>
 FFT_DEV void copy_elem(const fftk_copy_params& p, uint64_t gid)

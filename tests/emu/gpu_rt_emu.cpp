@@ -215,6 +215,23 @@ int fftrt_launch_copy(const struct fftk_copy_params* p, int precision, void*)
     return 0;
 }
 
+int fftrt_launch_callback_copy(const struct fftk_cb_params* p, int precision, int complex_elems, void*)
+{
+    uint64_t total = (uint64_t)p->len[0] * p->len[1] * p->len[2] * p->batch;
+    for(uint64_t g = 0; g < total; ++g)
+    {
+        if(precision == 0 && complex_elems)
+            callback_elem<float2>(*p, g);
+        else if(precision == 0)
+            callback_elem<float>(*p, g);
+        else if(complex_elems)
+            callback_elem<double2>(*p, g);
+        else
+            callback_elem<double>(*p, g);
+    }
+    return 0;
+}
+
 int fftrt_has_big32k(void)
 {
     return 0;

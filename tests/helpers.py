@@ -129,7 +129,7 @@ def make_input(kind, lengths, batch, seed=1):
 def run_transform(lib, backend, kind, lengths, batch, precision, inplace=False, in_type=None,
                   out_type=None, in_strides=None, in_dist=0, out_strides=None, out_dist=0,
                   in_offsets=None, out_offsets=None, scale=None, x=None, seed=1, use_work_buffer=True,
-                  stream=None, return_buffers=False):
+                  stream=None, return_buffers=False, info_hook=None):
     """Runs one plan; returns (output as (batch, n_out) float64/complex128, reference input used)."""
     rt = np.float32 if precision == B.SINGLE else np.float64
     dit, dot = default_types(kind)
@@ -193,6 +193,7 @@ def run_transform(lib, backend, kind, lengths, batch, precision, inplace=False, 
         info.set_work_buffer(backend.ptr(work), wb)
     if stream is not None:
         info.set_stream(stream)
+    hook_state = info_hook(info, backend, rt) if info_hook else None  # kept alive until the result is read
     plan.execute([backend.ptr(b) for b in in_bufs],
                  None if inplace else [backend.ptr(b) for b in out_bufs], info)
     backend.sync()
@@ -214,6 +215,7 @@ def run_transform(lib, backend, kind, lengths, batch, precision, inplace=False, 
                 mask[starts + k] = True
             touched.append((backend.to_numpy(b), mask))
         return y, x, touched
+    del hook_state
     plan.destroy()
     return y, x
 

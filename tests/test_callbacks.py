@@ -1,0 +1,103 @@
+"""Load/store callbacks (reference library/include/rocfft/rocfft.h:533-612): the callbacks of
+tests/cb scale every element on the way in and on the way out, so the result must equal
+s_load * s_store * transform(x), and an out-of-place transform must leave its input alone."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import helpers as H
+import rocfft_amd.binding as B
+from oracle import oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+S_LOAD, S_STORE = 0.75, -1.5
+
+CASES = [
+    (B.COMPLEX_FORWARD, [64], 3, B.SINGLE, {}),
+    (B.COMPLEX_INVERSE, [100, 6], 2, B.DOUBLE, {"inplace": True}),
+    (B.REAL_FORWARD, [128], 3, B.DOUBLE, {}),
+    (B.REAL_FORWARD, [30, 4], 2, B.SINGLE, {"inplace": True}),
+    (B.REAL_INVERSE, [64, 8], 2, B.SINGLE, {}),
+    (B.REAL_INVERSE, [15], 3, B.DOUBLE, {"inplace": True}),
+    (B.COMPLEX_FORWARD, [16384], 2, B.SINGLE, {}),
+    (B.COMPLEX_FORWARD, [97], 2, B.DOUBLE, {"in_strides": [2], "in_dist": 200, "out_strides": [3], "out_dist": 300,
+                                            "in_offsets": [5, 0], "out_offsets": [2, 0]}),
+]
+
+
+def callback_library(name):
+    path = os.path.join(ROOT, "tests", "cb", name)
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "tests", "cb")])
+    lib = ctypes.CDLL(path)
+    lib.cb_get.restype = ctypes.c_void_p
+    lib.cb_get.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    return lib
+
+
+def make_hook(cblib, kind, precision, which):
+    in_complex = kind != B.REAL_FORWARD
+    out_complex = kind != B.REAL_INVERSE
+
+    def hook(info, backend, rt):
+        keep = []
+        for use, is_store, cplx, value in (("load" in which, 0, in_complex, S_LOAD),
+                                           ("store" in which, 1, out_complex, S_STORE)):
+            if not use:
+                continue
+            fn = cblib.cb_get(is_store, 1 if cplx else 0, 1 if precision == B.DOUBLE else 0)
+            assert fn
+            data = backend.alloc(64)
+            backend.scatter(data, rt, np.array([0]), np.array([value], dtype=rt))
+            keep.append(data)
+            (info.set_store_callback if is_store else info.set_load_callback)(fn, backend.ptr(data))
+        return keep
+    return hook
+
+
+def check_case(lib, backend, cblib, kind, lengths, batch, precision, kw, which):
+    y, x = H.run_transform(lib, backend, kind, lengths, batch, precision,
+                           info_hook=make_hook(cblib, kind, precision, which), **kw)
+    factor = (S_LOAD if "load" in which else 1.0) * (S_STORE if "store" in which else 1.0)
+    ref = H.reference(kind, lengths, batch, x, precision) * factor
+    l2, linf = orc.rel_norms(y.reshape(-1), ref.reshape(-1))
+    tol = H.tolerance(precision)
+    assert l2 <= tol and linf <= tol, (kind, lengths, precision, kw, which, l2, linf)
+
+
+@pytest.mark.parametrize("which", ["load", "store", "load+store"])
+def test_callbacks_through_the_emulation(emu, which):
+    cblib = callback_library("libcb_host.so")
+    for kind, lengths, batch, precision, kw in CASES:
+        check_case(emu, H.HostBackend(), cblib, kind, lengths, batch, precision, kw, which)
+
+
+def test_callback_rules(emu):
+    info = B.ExecutionInfo(emu)
+    fn = (ctypes.c_void_p * 1)(1)
+    c = emu.c
+    # shared memory for callbacks is not supported (reference library/src/transform.cpp:80-81)
+    assert c.rocfft_execution_info_set_load_callback(info.handle, fn, None, 8) == B.STATUS_INVALID_ARG_VALUE
+    # planar arrays cannot be combined with callbacks
+    cblib = callback_library("libcb_host.so")
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [16], 1,
+                  B.PlanDescription(emu).set_data_layout(B.COMPLEX_PLANAR, B.COMPLEX_PLANAR), lib=emu)
+    info.set_load_callback(cblib.cb_get(0, 1, 0), None)
+    a = np.zeros(64, dtype=np.float32)
+    assert plan.execute_status([a.ctypes.data, a.ctypes.data], [a.ctypes.data, a.ctypes.data], info) == B.STATUS_FAILURE
+    # clearing the callback makes the same info usable again
+    info.set_load_callback(None)
+    re, im, ore, oim = (np.zeros(16, dtype=np.float32) for _ in range(4))
+    assert plan.execute_status([re.ctypes.data, im.ctypes.data], [ore.ctypes.data, oim.ctypes.data], info) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", ["load", "store", "load+store"])
+def test_callbacks_on_the_gpu(gpu_lib, which):
+    cblib = callback_library("libcb_device.so")
+    for kind, lengths, batch, precision, kw in CASES:
+        print("callback case", kind, lengths, precision, kw, which, flush=True)
+        check_case(gpu_lib, H.TorchBackend(), cblib, kind, lengths, batch, precision, kw, which)
