@@ -190,9 +190,14 @@ ROCFFT_EXPORT rocfft_status rocfft_execution_info_set_work_buffer(rocfft_executi
 ROCFFT_EXPORT rocfft_status rocfft_execution_info_set_stream(rocfft_execution_info info,
                                                              void*                 stream);
 
-/* User load/store device callbacks (reference rocfft.h:568-612).  They need
-   run-time compiled kernels, which this library does not have: both return
-   rocfft_status_failure after validating their arguments. */
+/* User load/store device callbacks (reference rocfft.h:533-612):
+     T    load_cb (T* data, size_t offset, void* cbdata, void* sharedMem);
+     void store_cb(T* data, size_t offset, T element, void* cbdata, void* sharedMem);
+   T is the element type of the input (output) array, offset counts such elements from the
+   buffer pointer given to rocfft_execute.  cb_functions[0] / cb_data[0] are used (one
+   device); a null function clears the callback; shared_mem_bytes must be 0
+   (rocfft_status_invalid_arg_value otherwise).  An execute with callbacks fails for planar
+   arrays and during stream capture. */
 ROCFFT_EXPORT rocfft_status rocfft_execution_info_set_load_callback(rocfft_execution_info info,
                                                                     void** cb_functions,
                                                                     void** cb_data,
