@@ -41,6 +41,7 @@ struct rocfft_plan_t
     ExecPlan    exec;
     int         device = 0;
     std::string error;
+    bool        half_io = false; // half-precision arrays: the plan computes in single precision on scratch copies
 };
 
 struct rocfft_execution_info_t
@@ -323,7 +324,7 @@ struct TraceLine
     }
 };
 
-static std::string bench_command(const Problem& p)
+static std::string bench_command(const Problem& p, bool half_io)
 {
     std::ostringstream o;
     o << "rocfft-bench --length ";
@@ -333,7 +334,7 @@ static std::string bench_command(const Problem& p)
     if(p.placement == rocfft_placement_notinplace)
         o << "-o ";
     o << "-t " << (int)p.type << " --precision "
-      << (p.precision == rocfft_precision_double ? "double" : p.precision == rocfft_precision_half ? "half" : "single")
+      << (half_io ? "half" : p.precision == rocfft_precision_double ? "double" : "single")
       << " --itype " << (int)p.in_type << " --otype " << (int)p.out_type << " --istride ";
     for(size_t d = p.rank; d-- > 0;)
         o << p.istride[d] << " ";
@@ -395,11 +396,14 @@ rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement plac
         .arg("description", (const void*)description);
     try
     {
-        rocfft_plan_t* p  = new rocfft_plan_t;
-        rocfft_status  st = make_problem(p->prob, placement, transform_type, precision, dimensions,
-                                        lengths, number_of_transforms, description);
+        rocfft_plan_t* p = new rocfft_plan_t;
+        // half precision: same layouts, single-precision arithmetic on staged copies
+        p->half_io       = precision == rocfft_precision_half;
+        rocfft_status st = make_problem(p->prob, placement, transform_type,
+                                        p->half_io ? rocfft_precision_single : precision, dimensions, lengths,
+                                        number_of_transforms, description);
         if(st == rocfft_status_success && (g_layers & LOG_BENCH))
-            log_line(LOG_BENCH, bench_command(p->prob));
+            log_line(LOG_BENCH, bench_command(p->prob, p->half_io));
         if(st == rocfft_status_success)
         {
             int ndev = 0;
@@ -486,39 +490,50 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         if(pass_ms && fftrt_stream_capturing(stream))
             return rocfft_status_failure;
 
-        // Load/store callbacks: the input is copied into a scratch buffer of the same layout
-        // through the load callback, the plan runs on scratch buffers, and the result goes to
-        // the user's buffer through the store callback (two extra element-wise passes; the
-        // transform kernels themselves make no indirect calls).
-        void*      cb_in    = nullptr;
-        void*      cb_out   = nullptr;
-        const bool have_cb  = info && (info->load_cb || info->store_cb);
-        auto       cleanup  = [&]() {
-            if(own || cb_in || cb_out)
+        // Staging.  Load/store callbacks: the input is copied into a scratch buffer of the same
+        // layout through the load callback, the plan runs on scratch buffers, and the result
+        // goes to the user's buffer through the store callback (two extra element-wise
+        // passes; the transform kernels themselves make no indirect calls).  Half precision:
+        // the plan computes in single precision on scratch arrays of the same layout, filled
+        // from and written back to the user's half-precision arrays the same way.
+        void*      st_in[2]  = {nullptr, nullptr};
+        void*      st_out[2] = {nullptr, nullptr};
+        const bool have_cb   = info && (info->load_cb || info->store_cb);
+        const bool half_io   = plan->half_io;
+        const bool staging   = have_cb || half_io;
+        auto       cleanup   = [&]() {
+            if(own || staging)
                 fftrt_stream_sync(stream);
             if(own)
                 fftrt_free(work);
-            if(cb_in)
-                fftrt_free(cb_in);
-            if(cb_out && cb_out != cb_in)
-                fftrt_free(cb_out);
+            for(int i = 0; i < 2; ++i)
+            {
+                if(st_in[i])
+                    fftrt_free(st_in[i]);
+                if(st_out[i] && st_out[i] != st_in[i])
+                    fftrt_free(st_out[i]);
+            }
         };
         fftk_cb_params cin, cout;
         memset(&cin, 0, sizeof(cin));
         memset(&cout, 0, sizeof(cout));
-        bool in_complex = true, out_complex = true;
-        if(have_cb)
+        const bool in_planar = planar(pr.in_type), out_planar = planar(pr.out_type);
+        // elements of one buffer are complex pairs only for interleaved complex arrays
+        const bool in_complex  = pr.in_type != rocfft_array_type_real && !in_planar;
+        const bool out_complex = pr.out_type != rocfft_array_type_real && !out_planar;
+        const int  nin = in_planar ? 2 : 1, nout = out_planar ? 2 : 1;
+        bool       stage_in = false, stage_out = false;
+        if(staging)
         {
-            if(planar(pr.in_type) || planar(pr.out_type) || fftrt_stream_capturing(stream))
+            if((have_cb && (in_planar || out_planar || half_io)) || fftrt_stream_capturing(stream))
             {
                 cleanup();
                 return rocfft_status_failure;
             }
-            in_complex  = pr.in_type != rocfft_array_type_real;
-            out_complex = pr.out_type != rocfft_array_type_real;
-            const size_t scalar = pr.precision == rocfft_precision_double ? 8 : 4;
+            const size_t scalar = ep.precision ? 8 : 4; // of the scratch arrays
             auto         fill   = [&](fftk_cb_params& c, bool input) {
-                size_t extent = (input ? pr.ioffset[0] : pr.ooffset[0]) + 1;
+                size_t off0   = input ? std::max(pr.ioffset[0], pr.ioffset[1]) : std::max(pr.ooffset[0], pr.ooffset[1]);
+                size_t extent = off0 + 1;
                 for(size_t d = 0; d < 3; ++d)
                 {
                     size_t n = d < pr.rank ? pr.len[d] : 1;
@@ -529,53 +544,57 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
                     c.stride[d] = d < pr.rank ? (int64_t)(input ? pr.istride[d] : pr.ostride[d]) : 0;
                     extent += (n - 1) * (size_t)c.stride[d];
                 }
-                c.batch  = (uint32_t)pr.batch;
-                c.dist   = (int64_t)(input ? pr.idist : pr.odist);
-                c.offset = (int64_t)(input ? pr.ioffset[0] : pr.ooffset[0]);
+                c.batch = (uint32_t)pr.batch;
+                c.dist  = (int64_t)(input ? pr.idist : pr.odist);
                 extent += (pr.batch - 1) * (size_t)c.dist;
                 return extent * scalar * ((input ? in_complex : out_complex) ? 2 : 1);
             };
             const size_t in_bytes  = fill(cin, true);
             const size_t out_bytes = fill(cout, false);
-            const bool   stage_in  = ep.inplace || info->load_cb;
-            const bool   stage_out = ep.inplace || info->store_cb;
-            if(stage_in && fftrt_malloc(&cb_in, ep.inplace ? std::max(in_bytes, out_bytes) : in_bytes) != 0)
+            stage_in               = ep.inplace || half_io || info->load_cb;
+            stage_out              = ep.inplace || half_io || info->store_cb;
+            bool ok                = true;
+            for(int i = 0; i < nin && ok && stage_in; ++i)
+                ok = fftrt_malloc(&st_in[i], ep.inplace ? std::max(in_bytes, out_bytes) : in_bytes) == 0;
+            for(int i = 0; i < nout && ok && stage_out; ++i)
             {
-                cleanup();
-                return rocfft_status_failure;
+                if(ep.inplace)
+                    st_out[i] = st_in[i];
+                else
+                    ok = fftrt_malloc(&st_out[i], out_bytes) == 0;
             }
-            if(ep.inplace)
-                cb_out = cb_in;
-            else if(stage_out && fftrt_malloc(&cb_out, out_bytes) != 0)
-            {
-                cleanup();
-                return rocfft_status_failure;
-            }
-            if(stage_in)
+            for(int i = 0; i < nin && ok && stage_in; ++i)
             {
                 cin.store   = 0;
-                cin.user    = in[0];
-                cin.scratch = cb_in;
-                cin.fn      = info->load_cb;
-                cin.data    = info->load_cb_data;
-                if(fftrt_launch_callback_copy(&cin, ep.precision, in_complex ? 1 : 0, stream) != 0)
-                {
-                    cleanup();
-                    return rocfft_status_failure;
-                }
+                cin.offset  = (int64_t)pr.ioffset[i];
+                cin.user    = in[i];
+                cin.scratch = st_in[i];
+                cin.fn      = half_io ? nullptr : info->load_cb;
+                cin.data    = half_io ? nullptr : info->load_cb_data;
+                ok = (half_io ? fftrt_launch_half_copy(&cin, in_complex ? 1 : 0, stream)
+                              : fftrt_launch_callback_copy(&cin, ep.precision, in_complex ? 1 : 0, stream))
+                     == 0;
+            }
+            if(!ok)
+            {
+                cleanup();
+                return rocfft_status_failure;
             }
         }
-        void* run_in[2]  = {cb_in ? cb_in : in[0], in[1]};
-        void* run_out[2] = {cb_out ? cb_out : out[0], out[1]};
+        void* run_in[2]  = {stage_in ? st_in[0] : in[0], stage_in ? st_in[1] : in[1]};
+        void* run_out[2] = {stage_out ? st_out[0] : out[0], stage_out ? st_out[1] : out[1]};
         rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms);
-        if(st == rocfft_status_success && cb_out)
+        for(int i = 0; i < nout && st == rocfft_status_success && stage_out; ++i)
         {
             cout.store   = 1;
-            cout.user    = out[0];
-            cout.scratch = cb_out;
-            cout.fn      = info->store_cb;
-            cout.data    = info->store_cb_data;
-            if(fftrt_launch_callback_copy(&cout, ep.precision, out_complex ? 1 : 0, stream) != 0)
+            cout.offset  = (int64_t)pr.ooffset[i];
+            cout.user    = out[i];
+            cout.scratch = st_out[i];
+            cout.fn      = half_io ? nullptr : info->store_cb;
+            cout.data    = half_io ? nullptr : info->store_cb_data;
+            int rc       = half_io ? fftrt_launch_half_copy(&cout, out_complex ? 1 : 0, stream)
+                                   : fftrt_launch_callback_copy(&cout, ep.precision, out_complex ? 1 : 0, stream);
+            if(rc != 0)
                 st = rocfft_status_failure;
         }
         cleanup();
@@ -925,7 +944,10 @@ rocfft_status rocfft_amd_plan_describe(rocfft_result_placement placement,
     try
     {
         Problem       prob;
-        rocfft_status st = make_problem(prob, placement, transform_type, precision, dimensions, lengths,
+        // (half precision plans compute in single precision on staged copies)
+        rocfft_status st = make_problem(prob, placement, transform_type,
+                                        precision == rocfft_precision_half ? rocfft_precision_single : precision,
+                                        dimensions, lengths,
                                         number_of_transforms, description);
         if(st != rocfft_status_success)
             return st;

@@ -45,6 +45,8 @@ int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void*
 int fftrt_launch_copy(const struct fftk_copy_params* p, int precision, void* stream);
 // complex_elems: 1 = the array holds (re, im) pairs, 0 = real scalars
 int fftrt_launch_callback_copy(const struct fftk_cb_params* p, int precision, int complex_elems, void* stream);
+// the same copy between a half-precision user array and a single-precision scratch array
+int fftrt_launch_half_copy(const struct fftk_cb_params* p, int complex_elems, void* stream);
 
 // 1 when the one-workgroup 32768-point kernel is available in this runtime
 int fftrt_has_big32k(void);

@@ -84,6 +84,12 @@ __global__ __launch_bounds__(256) void callback_copy_kernel(const fftk_cb_params
     callback_elem<E>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
 }
 
+template <typename U, typename E>
+__global__ __launch_bounds__(256) void half_copy_kernel(const fftk_cb_params p)
+{
+    half_stage_elem<U, E>(p, (uint64_t)blockIdx.x * 256 + threadIdx.x);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void row_copy_kernel(const fftk_copy_params p)
 {
@@ -257,6 +263,21 @@ int fftrt_launch_callback_copy(const struct fftk_cb_params* p, int precision, in
         hipLaunchKernelGGL(callback_copy_kernel<double2>, g, b, 0, s, *p);
     else
         hipLaunchKernelGGL(callback_copy_kernel<double>, g, b, 0, s, *p);
+    return (int)hipGetLastError();
+}
+
+int fftrt_launch_half_copy(const struct fftk_cb_params* p, int complex_elems, void* stream)
+{
+    uint64_t total = (uint64_t)p->len[0] * p->len[1] * p->len[2] * p->batch;
+    uint64_t grid  = (total + 255) / 256;
+    if(grid == 0 || grid >= (1ull << 31))
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = (hipStream_t)stream;
+    dim3        g((uint32_t)grid), b(256);
+    if(complex_elems)
+        hipLaunchKernelGGL((half_copy_kernel<fft_half2, float2>), g, b, 0, s, *p);
+    else
+        hipLaunchKernelGGL((half_copy_kernel<fft_half, float>), g, b, 0, s, *p);
     return (int)hipGetLastError();
 }
 

@@ -582,6 +582,58 @@ FFT_DEV void real_pre_elem(const fftk_real_params& p, uint64_t gid)
     }
 }
 
+// half-precision storage types of the staging copies
+typedef _Float16 fft_half;
+struct fft_half2
+{
+    _Float16 x, y;
+};
+FFT_DEV float stage_cvt(fft_half v, float*)
+{
+    return (float)v;
+}
+FFT_DEV fft_half stage_cvt(float v, fft_half*)
+{
+    return (fft_half)v;
+}
+FFT_DEV float2 stage_cvt(fft_half2 v, float2*)
+{
+    float2 r;
+    r.x = (float)v.x;
+    r.y = (float)v.y;
+    return r;
+}
+FFT_DEV fft_half2 stage_cvt(float2 v, fft_half2*)
+{
+    fft_half2 r;
+    r.x = (fft_half)v.x;
+    r.y = (fft_half)v.y;
+    return r;
+}
+
+// one element of a half-precision staging copy: U is the user's element type (half or half
+// pair), E the scratch type (float or float pair)
+template <typename U, typename E>
+FFT_DEV void half_stage_elem(const fftk_cb_params& p, uint64_t gid)
+{
+    uint32_t i0 = (uint32_t)(gid % p.len[0]);
+    gid /= p.len[0];
+    uint32_t i1 = (uint32_t)(gid % p.len[1]);
+    gid /= p.len[1];
+    uint32_t i2 = (uint32_t)(gid % p.len[2]);
+    uint64_t b  = gid / p.len[2];
+    if(b >= p.batch)
+        return;
+    const size_t off = (size_t)(p.offset + (int64_t)b * p.dist + (int64_t)i0 * p.stride[0]
+                                + (int64_t)i1 * p.stride[1] + (int64_t)i2 * p.stride[2]);
+    U* user = static_cast<U*>(p.user);
+    E* scr  = static_cast<E*>(p.scratch);
+    if(!p.store)
+        scr[off] = stage_cvt(user[off], static_cast<E*>(nullptr));
+    else
+        user[off] = stage_cvt(scr[off], static_cast<U*>(nullptr));
+}
+
 // one element of a callback copy (fftk_cb_params); E is the element type of the array
 template <typename E>
 FFT_DEV void callback_elem(const fftk_cb_params& p, uint64_t gid)

@@ -232,6 +232,19 @@ int fftrt_launch_callback_copy(const struct fftk_cb_params* p, int precision, in
     return 0;
 }
 
+int fftrt_launch_half_copy(const struct fftk_cb_params* p, int complex_elems, void*)
+{
+    uint64_t total = (uint64_t)p->len[0] * p->len[1] * p->len[2] * p->batch;
+    for(uint64_t g = 0; g < total; ++g)
+    {
+        if(complex_elems)
+            half_stage_elem<fft_half2, float2>(*p, g);
+        else
+            half_stage_elem<fft_half, float>(*p, g);
+    }
+    return 0;
+}
+
 int fftrt_has_big32k(void)
 {
     return 0;

@@ -74,7 +74,9 @@ def test_status_codes(emu):
     h = ctypes.c_void_p()
     assert c.rocfft_plan_create(ctypes.byref(h), 1, 0, 0, 4, ln, 1, None) == B.STATUS_INVALID_DIMENSIONS
     assert c.rocfft_plan_create(ctypes.byref(h), 1, 0, 0, 0, ln, 1, None) == B.STATUS_INVALID_DIMENSIONS
-    assert c.rocfft_plan_create(ctypes.byref(h), 1, 0, B.HALF, 1, ln, 1, None) == B.STATUS_FAILURE
+    assert c.rocfft_plan_create(ctypes.byref(h), 1, 0, B.HALF, 1, ln, 1, None) == 0
+    c.rocfft_plan_destroy(h)
+    assert c.rocfft_plan_create(ctypes.byref(h), 1, 0, 7, 1, ln, 1, None) == B.STATUS_FAILURE  # no such precision
 
     def create(placement, kind, it, ot):
         d = B.PlanDescription(emu).set_data_layout(it, ot)
