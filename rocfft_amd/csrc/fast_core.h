@@ -104,7 +104,27 @@ FFT_DEV uint32_t fk_out_pos(uint32_t tt, int s, int k)
     return (b / c) * R * c + (b % c) + k * c;
 }
 
-template <typename T, typename Cfg, int P>
+// Where element j of the transform that the handle `w` names lives in LDS.  Rows of a tile:
+// w is the transform's index in the tile.  FkStrideAddr: w is the LDS index of element 0 and
+// the elements are STRIDE apart (the columns of a 2D tile held row by row).
+template <typename Cfg>
+struct FkRowAddr
+{
+    static FFT_DEV uint32_t at(uint32_t w, uint32_t j)
+    {
+        return fk_addr<Cfg>(w, j);
+    }
+};
+template <int STRIDE>
+struct FkStrideAddr
+{
+    static FFT_DEV uint32_t at(uint32_t base, uint32_t j)
+    {
+        return base + j * (uint32_t)STRIDE;
+    }
+};
+
+template <typename T, typename Cfg, int P, typename A = FkRowAddr<Cfg>>
 FFT_DEV void fk_read(const typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
                      typename cplx_of<T>::type* r)
 {
@@ -116,11 +136,11 @@ FFT_DEV void fk_read(const typename cplx_of<T>::type* lds, uint32_t w, uint32_t 
         {
 #pragma unroll
             for(int k = 0; k < R; ++k)
-                r[s * R + k] = lds[fk_addr<Cfg>(w, fk_in_pos<Cfg, P>(tt, s, k))];
+                r[s * R + k] = lds[A::at(w, fk_in_pos<Cfg, P>(tt, s, k))];
         }
 }
 
-template <typename T, typename Cfg, int P>
+template <typename T, typename Cfg, int P, typename A = FkRowAddr<Cfg>>
 FFT_DEV void fk_write(typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
                       const typename cplx_of<T>::type* r)
 {
@@ -132,12 +152,13 @@ FFT_DEV void fk_write(typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
         {
 #pragma unroll
             for(int k = 0; k < R; ++k)
-                lds[fk_addr<Cfg>(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
+                lds[A::at(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
         }
 }
 
+// tw_all: the stacked twiddle table of the schedule
 template <typename T, typename Cfg, int P>
-FFT_DEV void fk_compute(const fftk_params& p, uint32_t tt, typename cplx_of<T>::type* r)
+FFT_DEV void fk_compute(const void* tw_all, uint32_t tt, typename cplx_of<T>::type* r)
 {
     typedef typename cplx_of<T>::type C;
     constexpr int                     R = Cfg::radix(P);
@@ -150,7 +171,7 @@ FFT_DEV void fk_compute(const fftk_params& p, uint32_t tt, typename cplx_of<T>::
             continue;
         if(P > 0)
         {
-            const C* tw = static_cast<const C*>(p.tw) + Cfg::twoff(P);
+            const C* tw = static_cast<const C*>(tw_all) + Cfg::twoff(P);
             uint32_t bl = (tt + s * Cfg::TPT) % c;
 #pragma unroll
             for(int k = 1; k < R; ++k)
@@ -162,51 +183,59 @@ FFT_DEV void fk_compute(const fftk_params& p, uint32_t tt, typename cplx_of<T>::
 
 // all passes on register data; on entry r holds the inputs of pass 0, on exit
 // the outputs of the last pass (element (s,k) at fk_out_pos<last>)
-template <typename T, typename Cfg>
-__device__ __forceinline__ void fk_passes(const fftk_params& p, typename cplx_of<T>::type* lds,
-                                          uint32_t w, uint32_t tt, bool active,
-                                          typename cplx_of<T>::type* r, bool lds_busy)
+template <typename T, typename Cfg, typename A = FkRowAddr<Cfg>>
+__device__ __forceinline__ void fk_passes_tw(const void* tw_all, typename cplx_of<T>::type* lds,
+                                             uint32_t w, uint32_t tt, bool active,
+                                             typename cplx_of<T>::type* r, bool lds_busy)
 {
 #define FK_SYNC() __syncthreads()
     if(active)
-        fk_compute<T, Cfg, 0>(p, tt, r);
+        fk_compute<T, Cfg, 0>(tw_all, tt, r);
     if constexpr(Cfg::NP > 1)
     {
         if(lds_busy)
             FK_SYNC();
         if(active)
-            fk_write<T, Cfg, 0>(lds, w, tt, r);
+            fk_write<T, Cfg, 0, A>(lds, w, tt, r);
         FK_SYNC();
         if(active)
         {
-            fk_read<T, Cfg, 1>(lds, w, tt, r);
-            fk_compute<T, Cfg, 1>(p, tt, r);
+            fk_read<T, Cfg, 1, A>(lds, w, tt, r);
+            fk_compute<T, Cfg, 1>(tw_all, tt, r);
         }
     }
     if constexpr(Cfg::NP > 2)
     {
         FK_SYNC();
         if(active)
-            fk_write<T, Cfg, 1>(lds, w, tt, r);
+            fk_write<T, Cfg, 1, A>(lds, w, tt, r);
         FK_SYNC();
         if(active)
         {
-            fk_read<T, Cfg, 2>(lds, w, tt, r);
-            fk_compute<T, Cfg, 2>(p, tt, r);
+            fk_read<T, Cfg, 2, A>(lds, w, tt, r);
+            fk_compute<T, Cfg, 2>(tw_all, tt, r);
         }
     }
     if constexpr(Cfg::NP > 3)
     {
         FK_SYNC();
         if(active)
-            fk_write<T, Cfg, 2>(lds, w, tt, r);
+            fk_write<T, Cfg, 2, A>(lds, w, tt, r);
         FK_SYNC();
         if(active)
         {
-            fk_read<T, Cfg, 3>(lds, w, tt, r);
-            fk_compute<T, Cfg, 3>(p, tt, r);
+            fk_read<T, Cfg, 3, A>(lds, w, tt, r);
+            fk_compute<T, Cfg, 3>(tw_all, tt, r);
         }
     }
+}
+
+template <typename T, typename Cfg>
+__device__ __forceinline__ void fk_passes(const fftk_params& p, typename cplx_of<T>::type* lds,
+                                          uint32_t w, uint32_t tt, bool active,
+                                          typename cplx_of<T>::type* r, bool lds_busy)
+{
+    fk_passes_tw<T, Cfg>(p.tw, lds, w, tt, active, r, lds_busy);
 }
 
 // Lean path: both sides are interleaved complex arrays whose element offsets inside a

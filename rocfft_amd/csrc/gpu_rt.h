@@ -48,6 +48,14 @@ int fftrt_launch_callback_copy(const struct fftk_cb_params* p, int precision, in
 // the same copy between a half-precision user array and a single-precision scratch array
 int fftrt_launch_half_copy(const struct fftk_cb_params* p, int complex_elems, void* stream);
 
+// One-workgroup 2D kernel for small nA x nB complex transforms (nA the unit-stride dimension):
+// fftrt_fast2d_info returns 0 when there is none for these sizes, else 1 and the two pass
+// schedules, their threads per transform and the LDS pitch between rows.  The launch takes
+// p->n = nA, p->n2 = nB, p->W transforms per workgroup, p->tw / p->tw2 the twiddle tables.
+int fftrt_fast2d_info(uint32_t nA, uint32_t nB, uint32_t* radixA, uint32_t* nfA, uint32_t* radixB,
+                      uint32_t* nfB, uint32_t* tptA, uint32_t* tptB, uint32_t* pitchA);
+int fftrt_launch_fast2d(const struct fftk_params* p, int precision, uint32_t grid, size_t lds_bytes, void* stream);
+
 // 1 when the one-workgroup 32768-point kernel is available in this runtime
 int fftrt_has_big32k(void);
 int fftrt_launch_big32k(const struct fftk_big_params* p, void* stream);

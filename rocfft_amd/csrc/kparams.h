@@ -66,6 +66,7 @@ struct fftk_params
     uint32_t lean;       // fast kernel: plain interleaved complex in and out, strides below in
                          // complex elements fit 32 bits: branch-free addressing path
     uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
+    uint32_t n2;       // fused 2D kernel: length of the second (strided) dimension; tw2: its twiddles
     uint32_t stage_io; // lean path: move the tile between global memory and LDS with consecutive
                        // lanes on consecutive elements (transforms too short for coalesced
                        // register loads)
@@ -86,6 +87,7 @@ struct fftk_params
     void*       out1;
     // tables
     const void* tw;        // stacked per-pass twiddles
+    const void* tw2; // fused 2D kernel: stacked twiddles of the second dimension
     const void* ltw;       // two-level table for W_L^u: lo[0 .. 1<<ltw_shift), then hi[]
     uint32_t    ltw_shift; //
     uint32_t    aux_dim;   // which index is q: 0 none, 1 tile, 2/3/4 outer 0/1/2

@@ -1615,6 +1615,126 @@ static void emit_big(Builder& b, uint32_t mode, const std::vector<Other>& others
     b.plan->passes.push_back(rec);
 }
 
+// Dimensions 0 and 1 of a complex transform in one kernel, when both are small powers of two
+// and every 2D slice is a contiguous block on both sides.  Returns false (nothing emitted) when
+// the runtime has no such kernel for these sizes or the layout does not fit.
+static const bool g_use_2d = !getenv("ROCFFT_AMD_NO_2D");
+
+static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t batch, const View& in,
+                          const View& out, int dir, double scale, bool has_scale)
+{
+    if(!g_use_fast || !g_use_2d || rank < 2)
+        return false;
+    const size_t nA = len[0], nB = len[1], esize = b.esize;
+    uint32_t     ra[4], rb[4], nfa = 0, nfb = 0, tpta = 0, tptb = 0, pitch = 0;
+    if(nA > 64 || nB > 64
+       || !fftrt_fast2d_info((uint32_t)nA, (uint32_t)nB, ra, &nfa, rb, &nfb, &tpta, &tptb, &pitch))
+        return false;
+    auto plain = [](const IoRef& io) { return !io.planar && io.im_delta == 1 && io.off0 % 2 == 0; };
+    if(!plain(in.io) || !plain(out.io))
+        return false;
+    if(in.stride[0] != 2 || out.stride[0] != 2 || in.stride[1] != 2 * (int64_t)nA
+       || out.stride[1] != 2 * (int64_t)nA)
+        return false;
+    // the axes that enumerate the 2D slices: dimension 2 (if any) and the batch
+    std::vector<Axis> ax;
+    if(rank == 3 && len[2] > 1)
+        ax.push_back({(uint32_t)len[2], in.stride[2], out.stride[2], false});
+    if(batch > 1)
+        ax.push_back({(uint32_t)batch, in.stride[3], out.stride[3], false});
+    for(const Axis& a : ax)
+        if(a.is % 2 || a.os % 2 || a.is <= 0 || a.os <= 0)
+            return false;
+    // merge when the batch continues dimension 2
+    if(ax.size() == 2 && ax[0].is * (int64_t)ax[0].cnt == ax[1].is && ax[0].os * (int64_t)ax[0].cnt == ax[1].os
+       && (uint64_t)ax[0].cnt * ax[1].cnt < (1ull << 31))
+    {
+        ax[0].cnt *= ax[1].cnt;
+        ax.pop_back();
+    }
+    Axis tile = {1, 2 * (int64_t)(nA * nB), 2 * (int64_t)(nA * nB), false};
+    if(!ax.empty())
+    {
+        size_t t = (ax.size() == 2 && ax[1].is < ax[0].is) ? 1 : 0;
+        tile     = ax[t];
+        ax.erase(ax.begin() + (long)t);
+    }
+    const size_t tp       = nB * (size_t)pitch; // LDS elements per transform
+    const size_t max_elem = esize == 8 ? 4096 : 2048;
+    uint32_t     tpx      = (uint32_t)std::max(nB * tpta, nA * tptb);
+    uint32_t     K        = floor_pow2(std::max<size_t>(1, max_elem / (nA * nB)));
+    K                     = std::min(K, floor_pow2(std::max<uint32_t>(1, 256 / tpx)));
+    K                     = std::min(K, ceil_pow2(tile.cnt));
+    if(K * tpx > 512 || K * tp * esize > 64 * 1024)
+        return false;
+    if((uint64_t)K * (uint64_t)(tile.is / 2) >= (1ull << 31) || (uint64_t)K * (uint64_t)(tile.os / 2) >= (1ull << 31))
+        return false;
+
+    PassRec rec;
+    rec.kind = PASS_2D;
+    rec.src  = in.io;
+    rec.dst  = out.io;
+    fftk_params& k = rec.kp;
+    memset(&k, 0, sizeof(k));
+    k.n  = (uint32_t)nA;
+    k.n2 = (uint32_t)nB;
+    k.nf = nfa;
+    std::vector<uint32_t> va(ra, ra + nfa), vb(rb, rb + nfb);
+    for(uint32_t i = 0; i < nfa; ++i)
+        k.radix[i] = ra[i];
+    uint32_t twoff_a[FFTK_MAX_PASSES], twoff_b[FFTK_MAX_PASSES];
+    TablePtr twa = stacked_twiddles(va, b.precision, b.dry, twoff_a);
+    TablePtr twb = stacked_twiddles(vb, b.precision, b.dry, twoff_b);
+    k.tw         = twa->dptr;
+    k.tw2        = twb->dptr;
+    rec.tables.push_back(twa);
+    rec.tables.push_back(twb);
+    k.T        = tpta;
+    k.W        = K;
+    k.wshift   = log2u(K);
+    k.pitch    = pitch;
+    k.padshift = PADSHIFT;
+    k.tile_cnt = tile.cnt;
+    k.w_is     = tile.is;
+    k.w_os     = tile.os;
+    k.w_is_c   = (uint32_t)(tile.is / 2);
+    k.w_os_c   = (uint32_t)(tile.os / 2);
+    for(int i = 0; i < 3; ++i)
+    {
+        k.oc[i]   = 1;
+        k.o_is[i] = k.o_os[i] = 0;
+    }
+    for(size_t i = 0; i < ax.size(); ++i)
+    {
+        k.oc[i]   = ax[i].cnt;
+        k.o_is[i] = ax[i].is;
+        k.o_os[i] = ax[i].os;
+    }
+    k.nthreads    = (K * tpx + 63) / 64 * 64;
+    uint64_t grid = (uint64_t)((tile.cnt + K - 1) / K) * k.oc[0] * k.oc[1] * k.oc[2];
+    if(grid == 0 || grid >= (1ull << 31))
+        return false;
+    rec.grid = k.grid = (uint32_t)grid;
+    rec.lds           = K * tp * esize;
+    k.fast            = 1;
+    k.dir             = dir;
+    k.load_op         = FFTK_LOAD_COMPLEX;
+    k.store_op        = FFTK_STORE_COMPLEX;
+    k.n_in = k.n_out = (uint32_t)nA;
+    if(has_scale)
+    {
+        k.flags |= FFTK_F_SCALE;
+        k.scale = scale;
+    }
+    rec.vec_ok   = true;
+    rec.bytes_rw = 2.0 * (double)(nA * nB) * tile.cnt * k.oc[0] * k.oc[1] * k.oc[2] * (double)esize;
+    std::ostringstream note;
+    note << "2D fft " << nA << "x" << nB << " in one workgroup";
+    rec.note = note.str();
+    b.plan->passes.push_back(rec);
+    return true;
+}
+
 // element-wise copy of `cnt` elements per row between two array kinds (fftk_copy_params)
 static void emit_copy(Builder& b, uint32_t cnt, const std::vector<Other>& rows, int64_t s_s, const IoRef& src,
                       int64_t d_s, const IoRef& dst, const fftk_copy_params& proto, const char* what)
@@ -1957,7 +2077,10 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                 for(int d = 0; d < 4; ++d)
                     if(in.stride[d] != out.stride[d] && (d == 3 || (size_t)d < p.rank))
                         fail("in-place transforms need identical input and output layouts");
-            for(size_t d = 0; d < p.rank; ++d)
+            size_t first = 0;
+            if(emit_fused_2d(b, p.len, p.rank, p.batch, in, out, dir, p.scale, p.has_scale && p.rank == 2))
+                first = 2; // dimensions 0 and 1 are done
+            for(size_t d = first; d < p.rank; ++d)
             {
                 const View& src = d == 0 ? in : out;
                 if(emit_dims_staged(b, p.len, p.rank, p.batch, d, src, out, dir,
@@ -2227,6 +2350,17 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
                 return rocfft_status_failure;
             rc = fftrt_launch_big32k(&q, stream);
         }
+        else if(rec.kind == PASS_2D)
+        {
+            fftk_params k = rec.kp;
+            k.in0         = s0;
+            k.in1         = s1;
+            k.out0        = d0;
+            k.out1        = d1;
+            if(!aligned(s0, plan.elem_bytes) || !aligned(d0, plan.elem_bytes))
+                return rocfft_status_failure;
+            rc = fftrt_launch_fast2d(&k, plan.precision, rec.grid, rec.lds, stream);
+        }
         else if(rec.kind == PASS_COPY)
         {
             fftk_copy_params c = rec.cp;
@@ -2331,6 +2465,9 @@ std::string ExecPlan::describe() const
             o << " threads 1024 grid " << r.grid << " lds 135296";
         else if(r.kind == PASS_COPY)
             o << " rows " << r.cp.rows0 << "x" << r.cp.rows1 << "x" << r.cp.rows2;
+        else if(r.kind == PASS_2D)
+            o << " tile " << r.kp.W << "x" << r.kp.n << "x" << r.kp.n2 << " threads " << r.kp.nthreads << " grid "
+              << r.grid << " lds " << r.lds;
         else
             o << " half " << r.rp.half << " rows " << r.rp.rows0 << "x" << r.rp.rows1 << "x"
               << r.rp.rows2;

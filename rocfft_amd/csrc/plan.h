@@ -59,7 +59,8 @@ enum PassKind
     PASS_REAL_POST = 1,
     PASS_REAL_PRE  = 2,
     PASS_BIG       = 3, // one-workgroup 32768-point single-precision kernel
-    PASS_COPY      = 4  // element-wise row copy between array kinds
+    PASS_COPY      = 4, // element-wise row copy between array kinds
+    PASS_2D        = 5  // one-workgroup small 2D complex transform (kp holds its parameters)
 };
 
 // where a pass finds one side of its data: buffer, planar or not, scalar offsets

@@ -245,6 +245,17 @@ int fftrt_launch_half_copy(const struct fftk_cb_params* p, int complex_elems, vo
     return 0;
 }
 
+// no one-workgroup 2D kernel in the emulation: such plans take the per-dimension passes here
+int fftrt_fast2d_info(uint32_t, uint32_t, uint32_t*, uint32_t*, uint32_t*, uint32_t*, uint32_t*, uint32_t*,
+                      uint32_t*)
+{
+    return 0;
+}
+int fftrt_launch_fast2d(const struct fftk_params*, int, uint32_t, size_t, void*)
+{
+    return 1;
+}
+
 int fftrt_has_big32k(void)
 {
     return 0;

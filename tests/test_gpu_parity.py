@@ -123,6 +123,23 @@ def test_multi_dim(gpu, lengths):
         H.check(lib, be, kind, lengths, 1, B.SINGLE, inplace=True)
 
 
+def test_small_2d_in_one_workgroup(gpu):
+    """8..64 x 8..64 complex transforms run as one kernel; also as the first two dimensions of a
+    3D transform, in place, with a scale factor, and with fewer transforms than a workgroup takes."""
+    lib, be = gpu
+    for a in (8, 16, 32, 64):
+        for b_ in (8, 16, 32, 64):
+            print("2d", a, b_, flush=True)
+            H.check(lib, be, B.COMPLEX_FORWARD, [a, b_], 37, B.SINGLE)
+            H.check(lib, be, B.COMPLEX_INVERSE, [a, b_], 5, B.DOUBLE, inplace=True, scale=0.5)
+            H.check(lib, be, B.COMPLEX_FORWARD, [a, b_, 6], 3, B.DOUBLE)
+            H.check(lib, be, B.COMPLEX_INVERSE, [a, b_], 1, B.SINGLE)
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [16, 16], 100, lib=lib)
+    assert [name for name, _ in plan.passes()] == ["2D fft 16x16 in one workgroup"]
+    # a layout the one-kernel path does not take (padded rows) still works, in two passes
+    H.check(lib, be, B.COMPLEX_FORWARD, [16, 16], 4, B.SINGLE, in_strides=[1, 20], in_dist=400)
+
+
 def test_large_square_2d(gpu):
     # both dimensions beyond the longest single-kernel length
     lib, be = gpu
