@@ -55,6 +55,13 @@ int fftrt_launch_half_copy(const struct fftk_cb_params* p, int complex_elems, vo
 int fftrt_fast2d_info(uint32_t nA, uint32_t nB, uint32_t* radixA, uint32_t* nfA, uint32_t* radixB,
                       uint32_t* nfB, uint32_t* tptA, uint32_t* tptB, uint32_t* pitchA);
 int fftrt_launch_fast2d(const struct fftk_params* p, int precision, uint32_t grid, size_t lds_bytes, void* stream);
+// The same for real transforms of 2L x nB points (p->n = L, the half length; p->half_tw its
+// post-/pre-processing twiddles): forward reads real rows and writes L+1 bins per row, inverse the
+// other way round.  `pitch` is the LDS pitch between the rows of L+1 bins.
+int fftrt_fast2d_real_info(uint32_t L, uint32_t nB, uint32_t* radixA, uint32_t* nfA, uint32_t* radixB,
+                           uint32_t* nfB, uint32_t* tptA, uint32_t* tptB, uint32_t* pitch);
+int fftrt_launch_fast2d_real(const struct fftk_params* p, int precision, int inverse, uint32_t grid,
+                             size_t lds_bytes, void* stream);
 
 // 1 when the one-workgroup 32768-point kernel is available in this runtime
 int fftrt_has_big32k(void);

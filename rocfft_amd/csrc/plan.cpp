@@ -1620,21 +1620,32 @@ static void emit_big(Builder& b, uint32_t mode, const std::vector<Other>& others
 // the runtime has no such kernel for these sizes or the layout does not fit.
 static const bool g_use_2d = !getenv("ROCFFT_AMD_NO_2D");
 
-static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t batch, const View& in,
+// mode 0: complex; 1: real forward (in = the real rows seen as pairs, out = Hermitian rows);
+// 2: real inverse (in = Hermitian rows, out = real pairs).  len[0] is the transform length of
+// dimension 0 (the real length for modes 1 and 2, which must be even).
+static bool emit_fused_2d(Builder& b, int mode, const size_t* len, size_t rank, size_t batch, const View& in,
                           const View& out, int dir, double scale, bool has_scale)
 {
     if(!g_use_fast || !g_use_2d || rank < 2)
         return false;
-    const size_t nA = len[0], nB = len[1], esize = b.esize;
+    if(mode != 0 && (len[0] % 2 || len[0] < 8))
+        return false;
+    const size_t nA = mode ? len[0] / 2 : len[0]; // complex points per row that the row phase transforms
+    const size_t nB = len[1], esize = b.esize;
+    const size_t rowlen = mode ? nA + 1 : nA;     // elements per row of the LDS tile
     uint32_t     ra[4], rb[4], nfa = 0, nfb = 0, tpta = 0, tptb = 0, pitch = 0;
-    if(nA > 64 || nB > 64
-       || !fftrt_fast2d_info((uint32_t)nA, (uint32_t)nB, ra, &nfa, rb, &nfb, &tpta, &tptb, &pitch))
+    if(nA > 64 || nB > 64)
+        return false;
+    int have = mode ? fftrt_fast2d_real_info((uint32_t)nA, (uint32_t)nB, ra, &nfa, rb, &nfb, &tpta, &tptb, &pitch)
+                    : fftrt_fast2d_info((uint32_t)nA, (uint32_t)nB, ra, &nfa, rb, &nfb, &tpta, &tptb, &pitch);
+    if(!have)
         return false;
     auto plain = [](const IoRef& io) { return !io.planar && io.im_delta == 1 && io.off0 % 2 == 0; };
     if(!plain(in.io) || !plain(out.io))
         return false;
-    if(in.stride[0] != 2 || out.stride[0] != 2 || in.stride[1] != 2 * (int64_t)nA
-       || out.stride[1] != 2 * (int64_t)nA)
+    // unit stride along dimension 0, whole complex elements between rows
+    if(in.stride[0] != 2 || out.stride[0] != 2 || in.stride[1] <= 0 || out.stride[1] <= 0 || in.stride[1] % 2
+       || out.stride[1] % 2 || in.stride[1] / 2 >= (1ll << 24) || out.stride[1] / 2 >= (1ll << 24))
         return false;
     // the axes that enumerate the 2D slices: dimension 2 (if any) and the batch
     std::vector<Axis> ax;
@@ -1652,7 +1663,7 @@ static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t bat
         ax[0].cnt *= ax[1].cnt;
         ax.pop_back();
     }
-    Axis tile = {1, 2 * (int64_t)(nA * nB), 2 * (int64_t)(nA * nB), false};
+    Axis tile = {1, in.stride[1] * (int64_t)nB, out.stride[1] * (int64_t)nB, false};
     if(!ax.empty())
     {
         size_t t = (ax.size() == 2 && ax[1].is < ax[0].is) ? 1 : 0;
@@ -1661,8 +1672,8 @@ static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t bat
     }
     const size_t tp       = nB * (size_t)pitch; // LDS elements per transform
     const size_t max_elem = esize == 8 ? 4096 : 2048;
-    uint32_t     tpx      = (uint32_t)std::max(nB * tpta, nA * tptb);
-    uint32_t     K        = floor_pow2(std::max<size_t>(1, max_elem / (nA * nB)));
+    uint32_t     tpx      = (uint32_t)std::max(nB * tpta, rowlen * tptb);
+    uint32_t     K        = floor_pow2(std::max<size_t>(1, max_elem / (rowlen * nB)));
     K                     = std::min(K, floor_pow2(std::max<uint32_t>(1, 256 / tpx)));
     K                     = std::min(K, ceil_pow2(tile.cnt));
     if(K * tpx > 512 || K * tp * esize > 64 * 1024)
@@ -1689,6 +1700,12 @@ static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t bat
     k.tw2        = twb->dptr;
     rec.tables.push_back(twa);
     rec.tables.push_back(twb);
+    if(mode)
+    {
+        TablePtr htw = half_twiddles(nA, b.precision, b.dry);
+        k.half_tw    = htw->dptr;
+        rec.tables.push_back(htw);
+    }
     k.T        = tpta;
     k.W        = K;
     k.wshift   = log2u(K);
@@ -1699,6 +1716,10 @@ static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t bat
     k.w_os     = tile.os;
     k.w_is_c   = (uint32_t)(tile.is / 2);
     k.w_os_c   = (uint32_t)(tile.os / 2);
+    k.t_is     = in.stride[1];
+    k.t_os     = out.stride[1];
+    k.t_is_c   = (uint32_t)(in.stride[1] / 2);  // complex elements between rows
+    k.t_os_c   = (uint32_t)(out.stride[1] / 2);
     for(int i = 0; i < 3; ++i)
     {
         k.oc[i]   = 1;
@@ -1718,18 +1739,20 @@ static bool emit_fused_2d(Builder& b, const size_t* len, size_t rank, size_t bat
     rec.lds           = K * tp * esize;
     k.fast            = 1;
     k.dir             = dir;
-    k.load_op         = FFTK_LOAD_COMPLEX;
-    k.store_op        = FFTK_STORE_COMPLEX;
+    k.load_op         = mode == 2 ? FFTK_LOAD_C2R_PRE : FFTK_LOAD_COMPLEX;
+    k.store_op        = mode == 1 ? FFTK_STORE_R2C_POST : FFTK_STORE_COMPLEX;
     k.n_in = k.n_out = (uint32_t)nA;
     if(has_scale)
     {
         k.flags |= FFTK_F_SCALE;
         k.scale = scale;
     }
-    rec.vec_ok   = true;
-    rec.bytes_rw = 2.0 * (double)(nA * nB) * tile.cnt * k.oc[0] * k.oc[1] * k.oc[2] * (double)esize;
+    rec.vec_ok         = true;
+    const double lines = (double)tile.cnt * k.oc[0] * k.oc[1] * k.oc[2];
+    rec.bytes_rw       = (mode ? (double)(nA + rowlen) : 2.0 * (double)nA) * (double)nB * lines * (double)esize;
     std::ostringstream note;
-    note << "2D fft " << nA << "x" << nB << " in one workgroup";
+    note << (mode == 1 ? "2D real forward fft " : mode == 2 ? "2D real inverse fft " : "2D fft ") << len[0] << "x" << nB
+         << " in one workgroup";
     rec.note = note.str();
     b.plan->passes.push_back(rec);
     return true;
@@ -2078,7 +2101,7 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                     if(in.stride[d] != out.stride[d] && (d == 3 || (size_t)d < p.rank))
                         fail("in-place transforms need identical input and output layouts");
             size_t first = 0;
-            if(emit_fused_2d(b, p.len, p.rank, p.batch, in, out, dir, p.scale, p.has_scale && p.rank == 2))
+            if(emit_fused_2d(b, 0, p.len, p.rank, p.batch, in, out, dir, p.scale, p.has_scale && p.rank == 2))
                 first = 2; // dimensions 0 and 1 are done
             for(size_t d = first; d < p.rank; ++d)
             {
@@ -2108,7 +2131,14 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
         {
             View hv = complex_view(out_buf, p.out_type, p.ostride, p.odist, p.ooffset, p.rank);
             bool last0 = p.rank == 1;
-            if(even && n0 >= 2)
+            // small dimensions 0 and 1: one kernel for both
+            size_t next_dim = 1;
+            if(even && p.rank >= 2
+               && emit_fused_2d(b, 1, p.len, p.rank, p.batch,
+                                realpair_view(BUF_IN, p.istride, p.idist, p.ioffset, p.rank), hv, -1, p.scale,
+                                p.has_scale && p.rank == 2))
+                next_dim = 2;
+            else if(even && n0 >= 2)
             {
                 uint64_t half = n0 / 2;
                 View     rv   = realpair_view(BUF_IN, p.istride, p.idist, p.ioffset, p.rank);
@@ -2171,7 +2201,7 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                                               p.scale, last0 && p.has_scale);
                 }
             }
-            for(size_t d = 1; d < p.rank; ++d)
+            for(size_t d = next_dim; d < p.rank; ++d)
             {
                 DimOps ops = d + 1 == p.rank ? scale_ops : DimOps();
                 emit_dim(b, p.len[d], hv.stride[d], hv.stride[d],
@@ -2184,9 +2214,18 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
         // (an out-of-place real inverse may overwrite its input: reference
         // rocfft.h:107-112, library/src/assignment_policy.cpp:601-606), then dimension 0
         View hv = complex_view(BUF_IN, p.in_type, p.istride, p.idist, p.ioffset, p.rank);
-        for(size_t d = p.rank; d-- > 1;)
+        for(size_t d = p.rank; d-- > 2;)
             emit_dim(b, p.len[d], hv.stride[d], hv.stride[d],
                      other_axes(hv, hv, hlen, p.rank, p.batch, d), hv.io, hv.io, +1, DimOps());
+        // small dimensions 1 and 0: one kernel for both (it does not write to its input)
+        if(even && p.rank >= 2
+           && emit_fused_2d(b, 2, p.len, p.rank, p.batch, hv,
+                            realpair_view(out_buf, p.ostride, p.odist, p.ooffset, p.rank), +1, p.scale,
+                            p.has_scale))
+            return rocfft_status_success;
+        if(p.rank >= 2)
+            emit_dim(b, p.len[1], hv.stride[1], hv.stride[1], other_axes(hv, hv, hlen, p.rank, p.batch, 1),
+                     hv.io, hv.io, +1, DimOps());
         if(even && n0 >= 2)
         {
             uint64_t half = n0 / 2;
@@ -2359,7 +2398,11 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             k.out1        = d1;
             if(!aligned(s0, plan.elem_bytes) || !aligned(d0, plan.elem_bytes))
                 return rocfft_status_failure;
-            rc = fftrt_launch_fast2d(&k, plan.precision, rec.grid, rec.lds, stream);
+            if(k.store_op == FFTK_STORE_R2C_POST || k.load_op == FFTK_LOAD_C2R_PRE)
+                rc = fftrt_launch_fast2d_real(&k, plan.precision, k.load_op == FFTK_LOAD_C2R_PRE ? 1 : 0, rec.grid,
+                                              rec.lds, stream);
+            else
+                rc = fftrt_launch_fast2d(&k, plan.precision, rec.grid, rec.lds, stream);
         }
         else if(rec.kind == PASS_COPY)
         {

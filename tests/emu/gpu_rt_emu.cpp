@@ -255,6 +255,15 @@ int fftrt_launch_fast2d(const struct fftk_params*, int, uint32_t, size_t, void*)
 {
     return 1;
 }
+int fftrt_fast2d_real_info(uint32_t, uint32_t, uint32_t*, uint32_t*, uint32_t*, uint32_t*, uint32_t*, uint32_t*,
+                           uint32_t*)
+{
+    return 0;
+}
+int fftrt_launch_fast2d_real(const struct fftk_params*, int, int, uint32_t, size_t, void*)
+{
+    return 1;
+}
 
 int fftrt_has_big32k(void)
 {

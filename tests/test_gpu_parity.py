@@ -140,6 +140,33 @@ def test_small_2d_in_one_workgroup(gpu):
     H.check(lib, be, B.COMPLEX_FORWARD, [16, 16], 4, B.SINGLE, in_strides=[1, 20], in_dist=400)
 
 
+def test_small_real_2d_in_one_workgroup(gpu):
+    """8..64 x 8..64 real transforms, both directions, run as one kernel (half-length rows, fused
+    pre/post-processing on the LDS tile, columns of the N/2+1 bins); also in place (padded rows),
+    as the first two dimensions of a 3D transform, and with a scale factor."""
+    lib, be = gpu
+    for a in (8, 16, 32, 64):
+        for b_ in (8, 16, 32, 64):
+            print("real 2d", a, b_, flush=True)
+            H.check(lib, be, B.REAL_FORWARD, [a, b_], 37, B.SINGLE)
+            H.check(lib, be, B.REAL_INVERSE, [a, b_], 37, B.DOUBLE)
+            H.check(lib, be, B.REAL_FORWARD, [a, b_], 5, B.DOUBLE, inplace=True, scale=0.5)
+            H.check(lib, be, B.REAL_INVERSE, [a, b_], 5, B.SINGLE, inplace=True, scale=0.25)
+            H.check(lib, be, B.REAL_FORWARD, [a, b_, 6], 3, B.SINGLE)
+            H.check(lib, be, B.REAL_INVERSE, [a, b_, 6], 3, B.DOUBLE)
+    plan = B.Plan(B.NOTINPLACE, B.REAL_INVERSE, B.SINGLE, [16, 16, 16], 10, lib=lib)
+    assert [name for name, _ in plan.passes()] == ["column fft n=16", "2D real inverse fft 16x16 in one workgroup"]
+    # an out-of-place 2D real inverse through the one-kernel path leaves its input alone
+    import torch
+    x = torch.view_as_complex(torch.rand((9, 32, 17, 2), device=be.dev) - 0.5).contiguous()
+    keep = x.clone()
+    y = torch.empty((9, 32, 32), device=be.dev)
+    plan = B.Plan(B.NOTINPLACE, B.REAL_INVERSE, B.SINGLE, [32, 32], 9, lib=lib)
+    plan.execute([x.data_ptr()], [y.data_ptr()])
+    torch.cuda.synchronize()
+    assert torch.equal(x, keep)
+
+
 def test_large_square_2d(gpu):
     # both dimensions beyond the longest single-kernel length
     lib, be = gpu
