@@ -268,7 +268,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     const bool                        inv  = p.dir > 0;
     const C*       src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
     C*             dst = reinterpret_cast<C*>(static_cast<T*>(p.out0) + c.obase);
-    const uint32_t q   = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+    const uint32_t q   = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
     C              r[Cfg::EPT];
     bool           lds_busy = false;
 
@@ -592,7 +592,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         r[s * RL + k] = lds[fk_addr<Cfg>(ow, ot + s * Cfg::TPT + k * CL)];
         }
     }
-    const uint32_t oq = p.aux_dim == 1 ? c.tile0 + ow : c.q_block;
+    const uint32_t oq = p.aux_dim == 1 ? (c.tile0 + ow) >> p.aux_shift : c.q_block;
     const uint32_t lo = ot * p.t_os_c + ow * p.w_os_c;
     if(ook)
     {
@@ -723,7 +723,7 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
     {
         // r holds the forward spectrum: multiply by the stored spectrum, exchange re/im
         // and run the passes again, which makes the second transform an inverse one
-        uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+        uint32_t q = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
         if(Cfg::NP > 1)
             __syncthreads();
         if(active)

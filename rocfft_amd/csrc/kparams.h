@@ -91,6 +91,7 @@ struct fftk_params
     const void* ltw;       // two-level table for W_L^u: lo[0 .. 1<<ltw_shift), then hi[]
     uint32_t    ltw_shift; //
     uint32_t    aux_dim;   // which index is q: 0 none, 1 tile, 2/3/4 outer 0/1/2
+    uint32_t    aux_shift; // aux_dim 1: q = tile index >> aux_shift (a faster plain axis was merged into the tile axis)
     const void* half_tw;   // e^{-2 pi i j/(2n)}, j in [0, n/2], for the real pre/post steps
     const void* chirp;     // Bluestein chirp e^{+i pi m^2/N}, m in [0, blu_n)
     uint32_t    blu_n;

@@ -426,7 +426,12 @@ static bool narrow_column_ok(uint64_t n, size_t elem_bytes, int64_t is, int64_t 
 {
     if(is <= 0 || os <= 0)
         return false;
-    const size_t run     = (size_t)widest_column_tile(n, elem_bytes) * elem_bytes;
+    const size_t wmax = widest_column_tile(n, elem_bytes);
+    // the tile spans everything that lies between two elements of the dimension: its rows are
+    // whole contiguous runs, however short
+    if(wmax > 0 && (int64_t)(2 * wmax) >= is && (int64_t)(2 * wmax) >= os)
+        return true;
+    const size_t run     = wmax * elem_bytes;
     const size_t scalar  = elem_bytes / 2;
     const bool   aligned = ((size_t)is * scalar) % 512 == 0 || ((size_t)os * scalar) % 512 == 0;
     return run >= 64 || (!aligned && run >= 32);
@@ -511,6 +516,7 @@ struct Axis
     uint32_t cnt;
     int64_t  is, os;
     bool     aux;
+    uint32_t aux_shift = 0; // aux axis with a faster plain axis merged in: table index = index >> aux_shift
 };
 
 struct TileSpec
@@ -582,11 +588,21 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         for(size_t i = 0; i < ax.size() && !merged; ++i)
             for(size_t j = 0; j < ax.size() && !merged; ++j)
             {
-                if(i == j || ax[i].aux || ax[j].aux)
+                if(i == j || ax[i].aux)
+                    continue;
+                // a plain axis may also merge into the table-indexed (aux) axis it continues into,
+                // when its length is a power of two: the table index is then the merged index
+                // shifted right
+                if(ax[j].aux && (ax[j].aux_shift || (ax[i].cnt & (ax[i].cnt - 1)) || ax[i].cnt < 2))
                     continue;
                 if(ax[i].is * (int64_t)ax[i].cnt == ax[j].is && ax[i].os * (int64_t)ax[i].cnt == ax[j].os
                    && (uint64_t)ax[i].cnt * ax[j].cnt < (1ull << 31))
                 {
+                    if(ax[j].aux)
+                    {
+                        ax[i].aux       = true;
+                        ax[i].aux_shift = log2u(ax[i].cnt);
+                    }
                     ax[i].cnt *= ax[j].cnt;
                     ax.erase(ax.begin() + (long)j);
                     merged = true;
@@ -643,6 +659,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     k.in_fast_tile  = (tile_axis.cnt > 1 && tile_axis.is < s.t_is) ? 1 : 0;
     k.out_fast_tile = (tile_axis.cnt > 1 && tile_axis.os < s.t_os) ? 1 : 0;
     k.aux_dim       = tile_axis.aux ? 1 : 0;
+    k.aux_shift     = tile_axis.aux ? tile_axis.aux_shift : 0;
     for(int i = 0; i < 3; ++i)
     {
         k.oc[i]   = 1;
@@ -654,7 +671,10 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         k.o_is[i] = ax[i].is;
         k.o_os[i] = ax[i].os;
         if(ax[i].aux)
-            k.aux_dim = 2 + (uint32_t)i;
+        {
+            k.aux_dim   = 2 + (uint32_t)i;
+            k.aux_shift = ax[i].aux_shift;
+        }
     }
 
     // work split
@@ -1920,6 +1940,13 @@ static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t 
         if(i != e && len[i] > 1 && (src.stride[i] < src.stride[e] || out.stride[i] < out.stride[e]))
             column = true;
     if(!column || !smooth(n) || plain_dim_is_single(n, true, esize, src.stride[e], out.stride[e]))
+        return false;
+    // the tiles of the staged passes are as wide as the rows below dimension e are long; with
+    // short rows the plain split is faster (its pass A merges the rows into wider tiles)
+    uint64_t below = 1;
+    for(size_t i = 0; i < e; ++i)
+        below *= len[i];
+    if(below < 64)
         return false;
     uint64_t n1, n0;
     split_length(n, esize, true, n1, n0);

@@ -55,7 +55,7 @@ FFT_DEV void tile_decode(const fftk_params& p, uint32_t bid, TileCtx<T>& c)
     c.obase = (int64_t)c.tile0 * p.w_os + (int64_t)c.oi[0] * p.o_os[0] + (int64_t)c.oi[1] * p.o_os[1]
               + (int64_t)c.oi[2] * p.o_os[2];
     // (no indexing of oi[] with a run-time value: that would push the context into scratch memory)
-    c.q_block = p.aux_dim == 2 ? c.oi[0] : p.aux_dim == 3 ? c.oi[1] : p.aux_dim == 4 ? c.oi[2] : 0;
+    c.q_block = (p.aux_dim == 2 ? c.oi[0] : p.aux_dim == 3 ? c.oi[1] : p.aux_dim == 4 ? c.oi[2] : 0) >> p.aux_shift;
 }
 
 FFT_DEV uint32_t lds_addr(const fftk_params& p, uint32_t w, uint32_t j)
@@ -135,7 +135,7 @@ FFT_DEV typename cplx_of<T>::type
     uint32_t idx = 0;
     if(ok && (p.flags & FFTK_F_CHIRP_LOAD))
     {
-        uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+        uint32_t q = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
         idx        = j * p.chirp_js + q * p.chirp_qs;
         ok         = idx < p.blu_n;
     }
@@ -321,7 +321,7 @@ FFT_DEV void tile_conv(const fftk_params&         p,
     tile_walk(p, tid, p.n, false, [&](uint32_t w, uint32_t j) {
         if(c.tile0 + w >= p.tile_cnt)
             return;
-        uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+        uint32_t q = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
         C        v = lds[lds_addr(p, w, j)];
         C        b = static_cast<const C*>(p.convb)[j + q * p.convb_qs];
         v          = c_mul(v, b);
@@ -353,7 +353,7 @@ FFT_DEV void emit_elem(const fftk_params& p, const TileCtx<T>& c, uint32_t w, ui
         return;
     if(inv)
         v = c_swap(v);
-    uint32_t q = p.aux_dim == 1 ? c.tile0 + w : c.q_block;
+    uint32_t q = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
     if(p.flags & FFTK_F_TWIDDLE_STORE)
     {
         C t = large_twiddle<T>(p, j * q);
