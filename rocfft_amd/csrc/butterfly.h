@@ -294,6 +294,50 @@ struct Butterfly<T, 13>
 };
 
 template <typename T>
+struct Butterfly<T, 17>
+{
+    typedef typename cplx_of<T>::type C;
+    static FFT_DEV void               run(C* r)
+    {
+        const T cs[17] = {(T)1.0,
+                          (T)9.32472229404355804573115891821563386e-1,
+                          (T)7.39008917220659115924534309872648106e-1,
+                          (T)4.45738355776538267396457549379486855e-1,
+                          (T)9.22683594633019952396511071545064804e-2,
+                          (T)-2.73662990072082863539077935436813432e-1,
+                          (T)-6.02634636379256389178588154986840622e-1,
+                          (T)-8.50217135729614152134143922949352058e-1,
+                          (T)-9.82973099683901778281948844855198716e-1,
+                          (T)-9.82973099683901778281948844855198716e-1,
+                          (T)-8.50217135729614152134143922949352058e-1,
+                          (T)-6.02634636379256389178588154986840622e-1,
+                          (T)-2.73662990072082863539077935436813432e-1,
+                          (T)9.22683594633019952396511071545064804e-2,
+                          (T)4.45738355776538267396457549379486855e-1,
+                          (T)7.39008917220659115924534309872648106e-1,
+                          (T)9.32472229404355804573115891821563386e-1};
+        const T sn[17] = {(T)0.0,
+                          (T)3.61241666187152948744714596183700164e-1,
+                          (T)6.73695643646557211712691912425694616e-1,
+                          (T)8.95163291355062322067016499753785457e-1,
+                          (T)9.95734176295034521871191178905481784e-1,
+                          (T)9.61825643172819070408796290731518550e-1,
+                          (T)7.98017227280239503332805112796261369e-1,
+                          (T)5.26432162877355800244607799140699566e-1,
+                          (T)1.83749517816570331574408839620727582e-1,
+                          (T)-1.83749517816570331574408839620727582e-1,
+                          (T)-5.26432162877355800244607799140699566e-1,
+                          (T)-7.98017227280239503332805112796261369e-1,
+                          (T)-9.61825643172819070408796290731518550e-1,
+                          (T)-9.95734176295034521871191178905481784e-1,
+                          (T)-8.95163291355062322067016499753785457e-1,
+                          (T)-6.73695643646557211712691912425694616e-1,
+                          (T)-3.61241666187152948744714596183700164e-1};
+        OddButterfly<T, 17>::run(r, cs, sn);
+    }
+};
+
+template <typename T>
 struct Butterfly<T, 8>
 {
     typedef typename cplx_of<T>::type C;

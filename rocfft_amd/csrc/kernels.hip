@@ -39,6 +39,7 @@ __device__ __forceinline__ void run_passes(const fftk_params&         p,
             FFTK_CASE(11)
             FFTK_CASE(13)
             FFTK_CASE(16)
+            FFTK_CASE(17)
 #undef FFTK_CASE
         default:
             __syncthreads();

@@ -12,7 +12,7 @@
 #include <stdint.h>
 
 #define FFTK_MAX_PASSES 12
-#define FFTK_REG_ELEMS 16 // complex values a thread keeps in registers per pass
+#define FFTK_REG_ELEMS 17 // complex values a thread keeps in registers per pass (one radix-17 butterfly)
 
 // how a tile element is fetched
 enum fftk_load_op

@@ -281,7 +281,7 @@ static bool factorize(uint64_t n, std::vector<uint32_t>& radix)
     radix.clear();
     if(n <= 1)
         return n == 1;
-    static const uint32_t odd[] = {13, 11, 7, 5, 3};
+    static const uint32_t odd[] = {17, 13, 11, 7, 5, 3};
     uint64_t              m     = n;
     for(uint32_t r : odd)
         while(m % r == 0)
@@ -1034,7 +1034,7 @@ static void split_three(uint64_t n, size_t esize, bool column, uint64_t& n2, uin
 static bool smooth(uint64_t n)
 {
     std::vector<uint32_t> r;
-    for(uint32_t p : {2u, 3u, 5u, 7u, 11u, 13u})
+    for(uint32_t p : {2u, 3u, 5u, 7u, 11u, 13u, 17u})
         while(n % p == 0)
             n /= p;
     return n == 1;

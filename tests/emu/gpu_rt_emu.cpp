@@ -52,6 +52,7 @@ void emu_passes(const fftk_params& p, typename cplx_of<T>::type* lds)
                     EMU_CASE(11)
                     EMU_CASE(13)
                     EMU_CASE(16)
+                    EMU_CASE(17)
 #undef EMU_CASE
                 default:
                     break;

@@ -229,13 +229,13 @@ def test_every_tile_fits_the_hardware(emu):
 
 def test_compiled_schedule_list_is_consistent(emu):
     """Every listed length has one schedule, its radices multiply to the length, the thread
-    count respects the register budget of 16 values per thread, and the planner uses it."""
+    count respects the register budget of 17 values per thread, and the planner uses it."""
     rows = H.fast_schedules()
     assert len(rows) == len({r[0] for r in rows}) and len(rows) > 200
     for n, radix, tf, td in rows:
         assert int(np.prod(radix)) == n and 1 <= len(radix) <= 4
-        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13, 16) for r in radix)
-        need = max(-(-(n // r) // (16 // r)) for r in radix)
+        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13, 16, 17) for r in radix)
+        need = max(-(-(n // r) // (17 // r)) for r in radix)
         for t in (tf, td):
             assert t == 0 or need <= t <= 1024
     for n, radix, tf, td in rows[::7]:
@@ -245,9 +245,9 @@ def test_compiled_schedule_list_is_consistent(emu):
 
 
 # the emulation runs the generic kernel on the schedules of the compiled kernels, composite
-# radices 6, 9 and 10 included
+# radices 6, 9 and 10 and the prime radix 17 included
 @pytest.mark.parametrize("n", [6, 9, 10, 12, 18, 36, 60, 81, 90, 100, 120, 125, 243, 250, 360, 480, 729,
-                               1000, 1536, 2187, 3000, 3645, 4000, 4032])
+                               1000, 1536, 2187, 3000, 3645, 4000, 4032, 17, 34, 289, 1156, 2040, 4046, 4080])
 def test_compiled_schedules_on_the_generic_kernel(emu, n):
     H.check(emu, HOST, B.COMPLEX_FORWARD, [n], 3, B.SINGLE)
     H.check(emu, HOST, B.COMPLEX_INVERSE, [n], 2, B.DOUBLE, inplace=True)
