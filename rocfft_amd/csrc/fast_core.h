@@ -242,8 +242,9 @@ __device__ __forceinline__ void fk_passes(const fftk_params& p, typename cplx_of
 // tile fit 32 bits.  Every address is a wave-uniform 64-bit base plus a 32-bit per-lane
 // element offset and there is no per-element branching on the operation kind, so the loads
 // of a thread issue back to back.  Covers plain passes, the large twiddle, scaling, the
-// Bluestein chirp on either side, convolution mode, the fused real pre/post-processing and
-// row-in/column-out passes.
+// Bluestein chirp on either side, convolution mode, the fused real pre/post-processing,
+// row-in/column-out passes and (odd lengths) real samples on one side with the half spectrum
+// on the other.
 template <typename T, typename Cfg>
 __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cplx_of<T>::type* lds,
                                                const TileCtx<T>& c, uint32_t tid, uint32_t w,
@@ -264,6 +265,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     // transforms whose lanes cover 16 contiguous bytes or less can go through LDS instead
     constexpr bool                    STAGE_OK = Cfg::TPT == 1 || Cfg::TPT * sizeof(C) <= 16;
     constexpr int                     STAGE_IT = (N + Cfg::TPT - 1) / Cfg::TPT;
+    // odd lengths also serve as odd-length real transforms (real samples on one side)
+    constexpr bool                    ODD_REAL = N % 2 == 1;
     const bool                        ok   = active && (c.tile0 + w < p.tile_cnt);
     const bool                        inv  = p.dir > 0;
     const C*       src = reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + c.ibase);
@@ -324,6 +327,55 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         if(active)
             fk_read<T, Cfg, 0>(lds, w, tt, r);
         lds_busy = true;
+    }
+    else if(ODD_REAL && p.load_op == FFTK_LOAD_REAL)
+    {
+        // odd-length real forward: real samples (strides in scalars), imaginary parts zero
+        const T*       srcr = static_cast<const T*>(p.in0) + c.ibase;
+        const uint32_t li   = tt * p.t_is_c + w * p.w_is_c;
+        if(ok)
+        {
+#pragma unroll
+            for(int s = 0; s < S0; ++s)
+#pragma unroll
+                for(int k = 0; k < R0; ++k)
+                {
+                    const T* pk = srcr + (uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c;
+                    if(fk_live<Cfg, 0>(tt, s))
+                    {
+                        C v;
+                        v.x           = pk[li];
+                        v.y           = 0;
+                        r[s * R0 + k] = inv ? c_swap(v) : v;
+                    }
+                }
+        }
+    }
+    else if(ODD_REAL && p.load_op == FFTK_LOAD_HERM_EXPAND)
+    {
+        // odd-length real inverse: bins 0..N/2 are stored, bin j > N/2 is the conjugate of bin
+        // N-j; the imaginary part of bin 0 is ignored
+        const uint32_t wo = w * p.w_is_c;
+        if(ok)
+        {
+#pragma unroll
+            for(int s = 0; s < S0; ++s)
+#pragma unroll
+                for(int k = 0; k < R0; ++k)
+                {
+                    const uint32_t j  = tt + s * Cfg::TPT + k * M0;
+                    const uint32_t jm = j <= (uint32_t)(N / 2) ? j : (uint32_t)N - j;
+                    if(fk_live<Cfg, 0>(tt, s))
+                    {
+                        C v = src[jm * p.t_is_c + wo];
+                        if(jm != j)
+                            v.y = -v.y;
+                        if(j == 0)
+                            v.y = 0;
+                        r[s * R0 + k] = inv ? c_swap(v) : v;
+                    }
+                }
+        }
     }
     else if(STAGE_OK && p.stage_io)
     {
@@ -651,6 +703,20 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     }
                 }
         }
+        else if(ODD_REAL && p.store_op == FFTK_STORE_REAL)
+        {
+            // real parts only (strides in scalars)
+            T* dstr = static_cast<T*>(p.out0) + c.obase;
+#pragma unroll
+            for(int s = 0; s < SL; ++s)
+#pragma unroll
+                for(int k = 0; k < RL; ++k)
+                {
+                    T* pk = dstr + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
+                    if(fk_live<Cfg, LAST>(ot, s))
+                        pk[lo] = r[s * RL + k].x;
+                }
+        }
         else
         {
 #pragma unroll
@@ -659,7 +725,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 for(int k = 0; k < RL; ++k)
                 {
                     C* pk = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
-                    if(fk_live<Cfg, LAST>(ot, s))
+                    // an odd-length real forward transform keeps the first n_out bins
+                    if(fk_live<Cfg, LAST>(ot, s) && (!ODD_REAL || ot + s * Cfg::TPT + k * CL < p.n_out))
                         pk[lo] = r[s * RL + k];
                 }
         }

@@ -215,7 +215,7 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
             return (int)hipErrorInvalidValue;
     if(cnt != p->nf)
         return (int)hipErrorInvalidValue;
-    fast_launch_fn fn = (vec && p->lean) ? e->lean : vec ? e->vec : e->scalar;
+    fast_launch_fn fn = p->lean ? e->lean : vec ? e->vec : e->scalar;
     if(!fn)
         return FFTRT_NO_FAST_VARIANT;
     return fn(p, grid, lds_bytes, stream);

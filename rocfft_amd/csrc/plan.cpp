@@ -276,12 +276,12 @@ static TablePtr chirp_table(uint64_t N, int precision, bool dry)
 // ---------------------------------------------------------------------------
 // factorisation
 
-static bool factorize(uint64_t n, std::vector<uint32_t>& radix)
+static bool factorize(uint64_t n, std::vector<uint32_t>& radix, bool composite = true)
 {
     radix.clear();
     if(n <= 1)
         return n == 1;
-    static const uint32_t odd[] = {17, 13, 11, 7, 5, 3};
+    static const uint32_t odd[] = {17, 13, 11, 7};
     uint64_t              m     = n;
     for(uint32_t r : odd)
         while(m % r == 0)
@@ -289,7 +289,17 @@ static bool factorize(uint64_t n, std::vector<uint32_t>& radix)
             radix.push_back(r);
             m /= r;
         }
-    uint32_t k = 0;
+    uint32_t k = 0, threes = 0, fives = 0;
+    while(m % 5 == 0)
+    {
+        ++fives;
+        m /= 5;
+    }
+    while(m % 3 == 0)
+    {
+        ++threes;
+        m /= 3;
+    }
     while(m % 2 == 0)
     {
         ++k;
@@ -297,6 +307,27 @@ static bool factorize(uint64_t n, std::vector<uint32_t>& radix)
     }
     if(m != 1)
         return false;
+    // composite butterflies save passes: 3*3 -> 9, then 5*2 -> 10 and 3*2 -> 6 while twos remain
+    for(; composite && threes >= 2; threes -= 2)
+        radix.push_back(9);
+    for(; fives > 0; --fives)
+        if(composite && k > 0)
+        {
+            radix.push_back(10);
+            --k;
+        }
+        else
+            radix.push_back(5);
+    for(; threes > 0; --threes)
+    {
+        if(composite && k > 0)
+        {
+            radix.push_back(6);
+            --k;
+        }
+        else
+            radix.push_back(3);
+    }
     // 2^k as radix-16 passes plus one or two smaller ones
     uint32_t a = k / 4, b = k % 4;
     std::vector<uint32_t> two;
@@ -359,7 +390,15 @@ static uint32_t kernel_schedule(uint64_t n, int precision, std::vector<uint32_t>
             return tpt;
         }
     }
-    if(!factorize(n, radix))
+    // composite radices save passes but want more threads; fall back to prime radices when
+    // that is what fits a workgroup
+    if(factorize(n, radix, true))
+    {
+        uint32_t T = threads_per_transform(n, radix);
+        if(T <= MAX_THREADS)
+            return T;
+    }
+    if(!factorize(n, radix, false))
         return 0;
     return threads_per_transform(n, radix);
 }
@@ -825,6 +864,39 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         }
     }
 
+    // odd-length real transforms on the same path: real samples in -> the first n/2+1 bins out,
+    // or those bins in (mirrored to the full spectrum on load) -> real samples out.  The real
+    // side is addressed in scalars, the complex side must be interleaved with even strides.
+    {
+        const bool fwd = s.load_op == FFTK_LOAD_REAL && s.store_op == FFTK_STORE_COMPLEX && k.n_in == k.n
+                         && k.n_out == k.n / 2 + 1;
+        const bool bwd = s.load_op == FFTK_LOAD_HERM_EXPAND && s.store_op == FFTK_STORE_REAL && k.n_in == k.n
+                         && k.n_out == k.n;
+        auto even = [](int64_t v) { return v % 2 == 0; };
+        bool cplx_ok = fwd ? (io_vec_ok(rec.dst, false) && even(k.t_os) && even(k.w_os))
+                           : (io_vec_ok(rec.src, false) && even(k.t_is) && even(k.w_is));
+        for(int i = 0; i < 3; ++i)
+            cplx_ok = cplx_ok && (fwd ? even(k.o_os[i]) : even(k.o_is[i]));
+        const bool real_ok = fwd ? !rec.src.planar : !rec.dst.planar;
+        if(k.fast && (fwd || bwd) && (k.n & 1u) && cplx_ok && real_ok && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0
+           && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
+        {
+            const int64_t ti = fwd ? k.t_is : k.t_is / 2, wi = fwd ? k.w_is : k.w_is / 2;
+            const int64_t to = fwd ? k.t_os / 2 : k.t_os, wo = fwd ? k.w_os / 2 : k.w_os;
+            uint64_t      in_span  = (uint64_t)(k.n + 1) * (uint64_t)ti + (uint64_t)W * (uint64_t)wi;
+            uint64_t      out_span = (uint64_t)(k.n + 1) * (uint64_t)to + (uint64_t)W * (uint64_t)wo;
+            if(in_span < (1ull << 28) && out_span < (1ull << 28))
+            {
+                rec.lean_ok = true;
+                rec.lean_real = true;
+                k.t_is_c    = (uint32_t)ti;
+                k.w_is_c    = (uint32_t)wi;
+                k.t_os_c    = (uint32_t)to;
+                k.w_os_c    = (uint32_t)wo;
+            }
+        }
+    }
+
     if(k.T > MAX_THREADS && !rec.lean_ok)
         fail("no kernel for a transform this long in this layout");
 
@@ -934,7 +1006,7 @@ static void split_length(uint64_t n, size_t esize, bool column, uint64_t& n1, ui
 
 static void split_length(uint64_t n, size_t esize, bool column, uint64_t& n1, uint64_t& n0);
 
-static bool factorize(uint64_t n, std::vector<uint32_t>& radix);
+static bool factorize(uint64_t n, std::vector<uint32_t>& radix, bool composite);
 
 static bool fast_kernel_exists(uint64_t n, size_t esize)
 {
@@ -2449,6 +2521,13 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             k.out1        = d1;
             bool vec = rec.vec_ok && aligned(s0, plan.elem_bytes) && aligned(d0, plan.elem_bytes);
             k.lean   = (rec.lean_ok && vec) ? 1 : 0;
+            if(rec.lean_real)
+            {
+                // the real side needs scalar alignment only
+                const bool in_ok  = aligned(s0, k.load_op == FFTK_LOAD_REAL ? plan.elem_bytes / 2 : plan.elem_bytes);
+                const bool out_ok = aligned(d0, k.store_op == FFTK_STORE_REAL ? plan.elem_bytes / 2 : plan.elem_bytes);
+                k.lean            = (in_ok && out_ok) ? 1 : 0;
+            }
             rc = fftrt_launch_tile(&k, plan.precision, vec ? 1 : 0, rec.grid, rec.lds, stream);
         }
         else

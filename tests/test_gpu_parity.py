@@ -68,6 +68,30 @@ def test_every_compiled_schedule(gpu):
         H.check(lib, be, B.COMPLEX_INVERSE, [n], 3, B.DOUBLE, inplace=True)
         H.check(lib, be, B.REAL_FORWARD, [2 * n], 3, B.SINGLE)
         H.check(lib, be, B.REAL_INVERSE, [2 * n], 3, B.DOUBLE)
+        if n % 2 == 1:
+            # odd-length real transforms run the same kernel with real samples on one side
+            H.check(lib, be, B.REAL_FORWARD, [n], 3, B.DOUBLE)
+            H.check(lib, be, B.REAL_INVERSE, [n], 3, B.SINGLE)
+
+
+def test_odd_real_layouts(gpu):
+    """Odd-length real transforms in one kernel: in place (padded rows), strided real side, a
+    scale factor, as dimension 0 of 2D/3D transforms, planar bins (no compiled variant: the
+    generic kernel), and a misaligned complex side."""
+    lib, be = gpu
+    for n in (9, 77, 153, 625, 1001, 2187, 4095):
+        H.check(lib, be, B.REAL_FORWARD, [n], 4, B.SINGLE, inplace=True, scale=0.5)
+        H.check(lib, be, B.REAL_INVERSE, [n], 4, B.DOUBLE, inplace=True, scale=0.25)
+        H.check(lib, be, B.REAL_FORWARD, [n], 3, B.DOUBLE, in_strides=[3], in_dist=3 * n + 1)
+        H.check(lib, be, B.REAL_INVERSE, [n], 3, B.SINGLE, out_strides=[2], out_dist=2 * n + 3)
+        H.check(lib, be, B.REAL_FORWARD, [n], 2, B.SINGLE, out_type=B.HERMITIAN_PLANAR)
+        H.check(lib, be, B.REAL_INVERSE, [n], 2, B.DOUBLE, in_type=B.HERMITIAN_PLANAR)
+        H.check(lib, be, B.REAL_FORWARD, [n], 2, B.SINGLE, in_offsets=[1, 0], out_offsets=[3, 0])
+        H.check(lib, be, B.REAL_INVERSE, [n], 2, B.SINGLE, in_offsets=[5, 0], out_offsets=[1, 0])
+    for lengths in ([7, 33, 5], [77, 27], [429, 64], [175, 35, 6], [25, 25, 25], [135, 512]):
+        for prec in (B.SINGLE, B.DOUBLE):
+            H.check(lib, be, B.REAL_FORWARD, lengths, 3, prec)
+            H.check(lib, be, B.REAL_INVERSE, lengths, 3, prec)
 
 
 def test_compiled_schedules_in_other_layouts(gpu):
