@@ -405,7 +405,10 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             if(p.flags & FFTK_F_CHIRP_LOAD)
             {
                 // samples beyond the signal read as zero; their loads are redirected to the
-                // first sample instead of being skipped, so that all loads stay in flight
+                // first element of the array instead of being skipped, so that all loads stay in
+                // flight (not to the first sample of this tile: the tile itself lies beyond the
+                // array when the table-indexed axis is longer than the signal)
+                const C*   first = reinterpret_cast<const C*>(static_cast<const T*>(p.in0));
                 const C*   chirp = static_cast<const C*>(p.chirp);
                 const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
                 C          ch[Cfg::EPT];
@@ -417,8 +420,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         const uint32_t j     = tt + s * Cfg::TPT + k * M0;
                         const uint32_t idx   = j * p.chirp_js + q * p.chirp_qs;
                         const bool     valid = idx < p.blu_n && fk_live<Cfg, 0>(tt, s);
-                        const uint32_t off   = valid ? j * p.t_is_c + w * p.w_is_c : 0u;
-                        r[s * R0 + k]        = src[off];
+                        const C*       pj    = valid ? src + (j * p.t_is_c + w * p.w_is_c) : first;
+                        r[s * R0 + k]        = *pj;
                         ch[s * R0 + k]       = chirp[valid ? idx : 0u];
                     }
 #pragma unroll

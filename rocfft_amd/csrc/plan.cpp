@@ -1437,6 +1437,16 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     // M = M1*M0: rows of length M0 are transformed, multiplied and transformed back by
     // one kernel, so that kernel gets the long factor; the strided passes get M1
     uint64_t M0 = 4096, M1 = M / M0;
+    {
+        // short strided passes make tiny workgroups: keep at least `floor` points in them
+        static const char* env   = getenv("ROCFFT_AMD_BLU_M1");
+        const uint64_t     floor = env ? (uint64_t)atoi(env) : (column ? 64 : 1);
+        if(M1 < floor && M / floor >= 64)
+        {
+            M1 = floor;
+            M0 = M / M1;
+        }
+    }
     while(M1 > 1 && !single_kernel_length(M1, esize))
         fail("Bluestein length too large");
     if(M1 < 2)
@@ -1446,18 +1456,44 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     // rows of the padded signals get a pitch that is not a power of two, so that the strided
     // column passes do not hammer one HBM channel
     const int64_t rowp = (int64_t)M0 + 16; // complex elements
-    b.need_blu(lines * M1 * (uint64_t)rowp);
-    std::vector<int64_t> pk = packed_strides(M1 * (uint64_t)rowp);
+    // The padded signals keep the axis order of the source, like the scratch array of the
+    // split: axes that run faster than this dimension (the columns of a strided dimension)
+    // stay innermost, so that a tile of neighbouring columns is contiguous there as well and
+    // all three passes are column passes over it; the other axes are packed outside.
+    std::vector<int64_t> pk(others.size(), 0);
+    int64_t              inner = 1;
+    {
+        std::vector<size_t> order(others.size());
+        for(size_t i = 0; i < others.size(); ++i)
+            order[i] = i;
+        std::sort(order.begin(), order.end(),
+                  [&](size_t x, size_t y) { return others[x].is < others[y].is; });
+        for(size_t i : order)
+            if(column && others[i].cnt > 1 && others[i].is < t_is)
+            {
+                pk[i] = 2 * inner;
+                inner *= others[i].cnt;
+            }
+        int64_t outer = (int64_t)M1 * rowp * 2 * inner;
+        for(size_t i : order)
+            if(pk[i] == 0)
+            {
+                pk[i] = outer;
+                outer *= others[i].cnt;
+            }
+        b.need_blu((size_t)(outer / 2));
+    }
+    const int64_t qS = 2 * inner; // scalar stride of one step along a padded signal
     {
         // Z1: chirp multiply + zero pad fused into the load of the column FFT over n1
         TileSpec s = base_spec();
         s.dir      = -1;
         s.n        = (uint32_t)M1;
         s.t_is     = (int64_t)M0 * t_is;
-        s.t_os     = rowp * 2;
+        s.t_os     = rowp * qS;
         s.src      = src;
         s.dst      = blu;
-        s.others.push_back({(uint32_t)M0, t_is, 2, true});
+        s.others.push_back({(uint32_t)M0, t_is, qS, true});
         add_others(s, true, false, pk);
         s.load_op         = ops.load_op;
         s.src_real_scalar = ops.src_real_scalar;
@@ -1476,9 +1512,9 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         TileSpec s = base_spec();
         s.dir      = -1;
         s.n        = (uint32_t)M0;
-        s.t_is = s.t_os = 2;
+        s.t_is = s.t_os = qS;
         s.src = s.dst = blu;
-        s.others.push_back({(uint32_t)M1, rowp * 2, rowp * 2, true});
+        s.others.push_back({(uint32_t)M1, rowp * qS, rowp * qS, true});
         add_others(s, false, false, pk);
         s.flags |= FFTK_F_CONV | FFTK_F_TWIDDLE_STORE;
         s.convb     = bs;
@@ -1493,11 +1529,11 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         TileSpec s = base_spec();
         s.dir      = +1;
         s.n        = (uint32_t)M1;
-        s.t_is     = rowp * 2;
+        s.t_is     = rowp * qS;
         s.t_os     = (int64_t)M0 * t_os;
         s.src      = blu;
         s.dst      = dst;
-        s.others.push_back({(uint32_t)M0, 2, t_os, true});
+        s.others.push_back({(uint32_t)M0, qS, t_os, true});
         add_others(s, false, true, pk);
         s.store_op        = ops.store_op;
         s.dst_real_scalar = ops.dst_real_scalar;

@@ -137,6 +137,20 @@ def test_long_odd_real(gpu, lengths):
     H.check(lib, be, B.REAL_INVERSE, lengths, 2, B.DOUBLE, inplace=True)
 
 
+@pytest.mark.parametrize("lengths", [[9, 2053], [64, 2053], [11, 2947], [40, 4099], [1155, 2084], [3, 5, 2311],
+                                     [6, 20011]])
+def test_bluestein_in_a_strided_dimension(gpu, lengths):
+    """A chirp-z dimension whose padded length needs the three-kernel form, behind a contiguous
+    dimension: the padded signals keep the columns innermost; the signal is shorter than the
+    row factor of the padded length in the first cases (loads of the padding must stay inside
+    the array)."""
+    lib, be = gpu
+    H.check(lib, be, B.COMPLEX_FORWARD, lengths, 2, B.SINGLE)
+    H.check(lib, be, B.COMPLEX_INVERSE, lengths, 1, B.DOUBLE, inplace=True)
+    H.check(lib, be, B.REAL_FORWARD, lengths, 2, B.DOUBLE)
+    H.check(lib, be, B.REAL_INVERSE, lengths, 1, B.SINGLE)
+
+
 @pytest.mark.parametrize("lengths", [[8, 8], [64, 64], [100, 30], [17, 19], [1024, 1024], [4096, 64], [64, 4096],
                                      [8, 8, 8], [16, 8, 4], [30, 20, 10], [128, 32, 8], [5, 7, 9], [8192, 4], [4, 8192], [64, 64, 64],
                                      [128, 128, 128], [512, 16, 16], [16, 512, 4], [8, 4, 512], [1, 8], [8, 1, 4]])
