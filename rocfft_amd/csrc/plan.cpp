@@ -1062,6 +1062,18 @@ static void split_two(uint64_t n, size_t esize, bool column, uint64_t& n1, uint6
         score += ratio;
         if(a < 8)
             score -= 1.0;
+        // a strided pass whose tile the thread count keeps narrow (many threads per transform)
+        // moves short runs
+        auto narrow = [&](uint64_t len) {
+            const size_t run = (size_t)widest_column_tile(len, esize) * esize;
+            return run < 64 ? 2.0 : run < COL_RUN_BYTES ? 1.0 : 0.0;
+        };
+        score -= narrow(a);
+        if(column)
+            score -= narrow(bq);
+        // ... and short runs a multiple of 512 bytes apart alias onto the same HBM channels
+        if(narrow(a) > 0 && (bq * esize) % 512 == 0)
+            score -= 0.5;
         if(score > best_score)
         {
             best_score = score;
