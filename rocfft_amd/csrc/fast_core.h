@@ -265,6 +265,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     // transforms whose lanes cover 16 contiguous bytes or less can go through LDS instead
     constexpr bool                    STAGE_OK = Cfg::TPT == 1 || Cfg::TPT * sizeof(C) <= 16;
     constexpr int                     STAGE_IT = (N + Cfg::TPT - 1) / Cfg::TPT;
+    constexpr int                     BINS_IT  = (N + 1 + Cfg::TPT - 1) / Cfg::TPT; // N+1 Hermitian bins per row
     // odd lengths also serve as odd-length real transforms (real samples on one side)
     constexpr bool                    ODD_REAL = N % 2 == 1;
     const bool                        ok   = active && (c.tile0 + w < p.tile_cnt);
@@ -284,6 +285,47 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         // has the unpaired bin N/2 besides.
         const C*       htw = static_cast<const C*>(p.half_tw);
         const uint32_t wo  = w * p.w_is_c;
+        bool           staged = false;
+        C              pa[STAGE_OK ? PAIR_IT : 1], pb[STAGE_OK ? PAIR_IT : 1], pm;
+        pm.x = pm.y = 0;
+        if constexpr(STAGE_OK)
+        {
+            if(p.stage_io)
+            {
+                // short transforms: consecutive lanes copy consecutive bins of the tile's rows
+                // (N+1 each) into LDS, then every thread takes its pairs from there
+                staged               = true;
+                const uint32_t total = p.W * (uint32_t)(N + 1);
+#pragma unroll
+                for(int i = 0; i < BINS_IT; ++i)
+                {
+                    const uint32_t e     = tid + i * p.nthreads;
+                    const uint32_t w_    = e / (uint32_t)(N + 1);
+                    const uint32_t j_    = e - w_ * (uint32_t)(N + 1);
+                    const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
+                    C              v     = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
+                    if(valid)
+                        lds[e] = v;
+                }
+                __syncthreads();
+                if(ok)
+                {
+                    const uint32_t row = w * (uint32_t)(N + 1);
+#pragma unroll
+                    for(int i = 0; i < PAIR_IT; ++i)
+                    {
+                        const uint32_t j = tt + i * Cfg::TPT;
+                        if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
+                            continue;
+                        pa[i] = lds[row + j];
+                        pb[i] = lds[row + (uint32_t)N - j];
+                    }
+                    if(N % 2 == 0 && tt == 0)
+                        pm = lds[row + N / 2];
+                }
+                __syncthreads();
+            }
+        }
         if(ok)
         {
 #pragma unroll
@@ -293,8 +335,17 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 const uint32_t jq = N - j;
                 if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
                     continue;
-                C              a  = src[j * p.t_is_c + wo];
-                C              bq = src[jq * p.t_is_c + wo];
+                C              a, bq;
+                if(STAGE_OK && staged)
+                {
+                    a  = pa[STAGE_OK ? i : 0];
+                    bq = pb[STAGE_OK ? i : 0];
+                }
+                else
+                {
+                    a  = src[j * p.t_is_c + wo];
+                    bq = src[jq * p.t_is_c + wo];
+                }
                 C              zj, zq;
                 if(j == 0)
                 {
@@ -316,7 +367,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             }
             if(N % 2 == 0 && tt == 0)
             {
-                C a = src[(N / 2) * p.t_is_c + wo];
+                C a = (STAGE_OK && staged) ? pm : src[(N / 2) * p.t_is_c + wo];
                 C z;
                 z.x                         = (T)2 * a.x;
                 z.y                         = (T)-2 * a.y;
@@ -531,6 +582,90 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         if(active)
             fk_write<T, Cfg, LAST>(lds, w, tt, r);
         __syncthreads();
+        if constexpr(STAGE_OK)
+        {
+            if(p.stage_io)
+            {
+                // short transforms: the bins go back to LDS as the image of the tile's output
+                // rows (N+1 bins each), which consecutive lanes then copy out
+                const C* htw = static_cast<const C*>(p.half_tw);
+                const T  sc  = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
+                C        zp[PAIR_IT], zq[PAIR_IT], zm;
+                zm.x = zm.y = 0;
+                if(ok)
+                {
+#pragma unroll
+                    for(int i = 0; i < PAIR_IT; ++i)
+                    {
+                        const uint32_t j = tt + i * Cfg::TPT;
+                        if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
+                            continue;
+                        zp[i] = lds[fk_addr<Cfg>(w, j)];
+                        zq[i] = lds[fk_addr<Cfg>(w, j == 0 ? 0u : (uint32_t)N - j)];
+                    }
+                    if(N % 2 == 0 && tt == 0)
+                        zm = lds[fk_addr<Cfg>(w, N / 2)];
+                }
+                __syncthreads();
+                if(ok)
+                {
+                    const uint32_t row = w * (uint32_t)(N + 1);
+#pragma unroll
+                    for(int i = 0; i < PAIR_IT; ++i)
+                    {
+                        const uint32_t j = tt + i * Cfg::TPT;
+                        if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
+                            continue;
+                        C o0, o1;
+                        if(j == 0)
+                        {
+                            o0.x = zp[i].x + zp[i].y;
+                            o0.y = 0;
+                            o1.x = zp[i].x - zp[i].y;
+                            o1.y = 0;
+                        }
+                        else
+                        {
+                            C t = htw[j];
+                            C u, v;
+                            u.x  = (T)0.5 * (zp[i].x + zq[i].x);
+                            u.y  = (T)0.5 * (zp[i].y + zq[i].y);
+                            v.x  = (T)0.5 * (zp[i].x - zq[i].x);
+                            v.y  = (T)0.5 * (zp[i].y - zq[i].y);
+                            o0.x = u.x + v.x * t.y + u.y * t.x;
+                            o0.y = v.y + u.y * t.y - v.x * t.x;
+                            o1.x = u.x - v.x * t.y - u.y * t.x;
+                            o1.y = -v.y + u.y * t.y - v.x * t.x;
+                        }
+                        o0.x *= sc;
+                        o0.y *= sc;
+                        o1.x *= sc;
+                        o1.y *= sc;
+                        lds[row + j]               = o0;
+                        lds[row + (uint32_t)N - j] = o1;
+                    }
+                    if(N % 2 == 0 && tt == 0)
+                    {
+                        C o;
+                        o.x              = zm.x * sc;
+                        o.y              = -zm.y * sc;
+                        lds[row + N / 2] = o;
+                    }
+                }
+                __syncthreads();
+                const uint32_t total = p.W * (uint32_t)(N + 1);
+#pragma unroll
+                for(int i = 0; i < BINS_IT; ++i)
+                {
+                    const uint32_t e  = tid + i * p.nthreads;
+                    const uint32_t w_ = e / (uint32_t)(N + 1);
+                    const uint32_t j_ = e - w_ * (uint32_t)(N + 1);
+                    if(e < total && c.tile0 + w_ < p.tile_cnt)
+                        dst[j_ * p.t_os_c + w_ * p.w_os_c] = lds[e];
+                }
+                return;
+            }
+        }
         if(ok)
         {
             const C*       htw = static_cast<const C*>(p.half_tw);

@@ -852,9 +852,13 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             {
                 rec.lean_ok = true;
                 // short transforms in unit-stride rows: coalesced tile copies through LDS
+                // (also the fused real pre/post-processing: rows of n+1 bins on that side)
+                const bool plain_ops = s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_COMPLEX;
+                const bool real_ops  = (s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_R2C_POST)
+                                      || (s.load_op == FFTK_LOAD_C2R_PRE && s.store_op == FFTK_STORE_COMPLEX);
                 if(!column && (k.T == 1 || ((size_t)k.T * esize <= 16 && k.n < 32)) && k.t_is == 2 && k.t_os == 2
-                   && s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_COMPLEX
-                   && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0 && k.n_in == k.n && k.n_out == k.n)
+                   && (plain_ops || real_ops) && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0 && k.n_in == k.n
+                   && k.n_out == k.n)
                     k.stage_io = 1;
                 k.t_is_c    = (uint32_t)(k.t_is / 2);
                 k.t_os_c    = (uint32_t)(k.t_os / 2);
