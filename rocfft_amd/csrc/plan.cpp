@@ -2296,8 +2296,11 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
                 auto     oth  = other_axes(rv, hv, p.len, p.rank, p.batch, 0);
                 if(big_eligible(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io))
                     emit_big(b, 1, oth, rv.io, hv.io, -1, p.scale, last0 && p.has_scale);
-                else if(single_kernel_length(half, b.esize))
+                else if(single_kernel_length(half, b.esize)
+                        && plain_dim_is_single(half, rv.stride[0] != 2, b.esize, rv.stride[0], hv.stride[0]))
                 {
+                    // (a half length that only the run-time-schedule kernel takes in one pass, but
+                    // whose two factors have compiled kernels, goes the unfused way below)
                     DimOps ops;
                     ops.store_op = FFTK_STORE_R2C_POST;
                     ops.half_tw  = half_twiddles(half, b.precision, b.dry);
@@ -2384,8 +2387,12 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
             auto     oth  = other_axes(hv, rv, p.len, p.rank, p.batch, 0);
             if(big_eligible(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io))
                 emit_big(b, 2, oth, hv.io, rv.io, +1, p.scale, p.has_scale);
-            else if(single_kernel_length(half, b.esize))
+            else if(single_kernel_length(half, b.esize)
+                    && (plan.inplace
+                        || plain_dim_is_single(half, rv.stride[0] != 2, b.esize, hv.stride[0], rv.stride[0])))
             {
+                // (out of place, a half length that only the run-time-schedule kernel takes in one
+                // pass but whose two factors have compiled kernels goes the unfused way below)
                 DimOps ops;
                 ops.load_op   = FFTK_LOAD_C2R_PRE;
                 ops.half_tw   = half_twiddles(half, b.precision, b.dry);
