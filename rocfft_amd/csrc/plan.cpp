@@ -1379,7 +1379,8 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
 
     // Bluestein chirp-z (reference: library/src/tree_node_bluestein.cpp:27-285,
     // library/src/rtc_bluestein_gen.cpp:170-380).  The convolution length M is the
-    // next power of two >= 2n-1; chirp and its spectrum are plan-time tables.
+    // next power of two >= 2n-1 or a shorter length of compiled kernels; chirp and its spectrum are
+    // plan-time tables.
     if(ops.store_op != FFTK_STORE_COMPLEX && ops.store_op != FFTK_STORE_REAL)
         fail("Bluestein cannot be combined with this real-transform step");
     if(ops.load_op == FFTK_LOAD_C2R_PRE)
@@ -1389,16 +1390,57 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     if(M >= (1ull << 31))
         fail("length too large");
     bool     conj_chirp = dir > 0;
-    // the whole convolution in one workgroup when M fits; strided data must keep a wide tile
-    bool one = column ? column_kernel_length(M, esize) : single_kernel_length(M, esize);
-    if(!one && column && single_kernel_length(M, esize) && M <= 4096)
-        one = true;
-    // single precision: M = 16384 still fits one workgroup of the wide compiled kernel
-    const bool wide_one = !one && !column && wide_kernel_length(M, esize);
+    const uint64_t Mpow2 = M;
+    auto one_kernel = [&](uint64_t m) {
+        // the whole convolution in one workgroup when m fits; strided data must keep a wide tile
+        bool ok = column ? column_kernel_length(m, esize) : single_kernel_length(m, esize);
+        if(!ok && column && single_kernel_length(m, esize) && m <= 4096)
+            ok = true;
+        return ok;
+    };
+    // Any length >= 2n-1 serves; a power of two can be almost twice that.  A shorter length made
+    // of compiled kernels is taken when it saves at least 30 % of the padded size (measured: no gain
+    // at 27 %; the kernels of other lengths are somewhat slower than those of powers of two).
+    uint64_t sM1 = 0, sM0 = 0; // factors of a shorter length for the three-kernel form
+    if(g_use_fast && !getenv("ROCFFT_AMD_BLU_POW2"))
+    {
+        const uint64_t need = 2 * N - 1, lim = Mpow2 / 10 * 7;
+        uint64_t       best = 0;
+        for(uint64_t m = need; m < lim && m <= 16384; ++m)
+            if(fast_kernel_exists(m, esize) && (one_kernel(m) || (!column && wide_kernel_length(m, esize))))
+            {
+                best = m;
+                break;
+            }
+        if(best == 0 && !one_kernel(Mpow2) && !(!column && wide_kernel_length(Mpow2, esize)))
+        {
+            // m = m1 * m0: m0 the row factor (one convolution kernel per row), m1 the strided one
+            const uint64_t lo0 = column ? 64 : 1024, lo1 = column ? 64 : 2;
+            for(uint64_t m0 = 4096; m0 >= lo0; --m0)
+            {
+                if(!fast_kernel_exists(m0, esize) || !single_kernel_length(m0, esize))
+                    continue;
+                uint64_t m1 = std::max<uint64_t>(lo1, (need + m0 - 1) / m0);
+                while(m1 * m0 < lim && !(fast_kernel_exists(m1, esize) && column_kernel_length(m1, esize)))
+                    ++m1;
+                if(m1 * m0 < lim && (best == 0 || m1 * m0 < best))
+                {
+                    best = m1 * m0;
+                    sM1  = m1;
+                    sM0  = m0;
+                }
+            }
+        }
+        if(best != 0)
+            M = best;
+    }
+    bool one = sM1 == 0 && one_kernel(M);
+    // single precision: the wide compiled kernels (up to M = 16384) still fit one workgroup
+    const bool wide_one = sM1 == 0 && !one && !column && wide_kernel_length(M, esize);
     // (checked before any table is computed: a chirp of 10^8 entries takes a minute)
     if(!one && !wide_one && (ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out))
         fail("odd-length real transforms of this size are not implemented");
-    if(!one && !single_kernel_length(M / 4096, esize))
+    if(!one && sM1 == 0 && !single_kernel_length(M / 4096, esize))
         fail("Bluestein length too large");
     TablePtr chirp      = chirp_table(N, b.precision, b.dry);
     double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
@@ -1446,6 +1488,18 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         catch(const PlanError&)
         {
             b.plan->passes.resize(mark);
+            if(M != Mpow2)
+            {
+                // this layout cannot use the wide kernel of the shorter length: back to the
+                // power of two, in one kernel if that fits
+                M     = Mpow2;
+                scale = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
+                if(one_kernel(M))
+                {
+                    emit_one();
+                    return;
+                }
+            }
         }
     }
     if(ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out)
@@ -1453,6 +1507,12 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     // M = M1*M0: rows of length M0 are transformed, multiplied and transformed back by
     // one kernel, so that kernel gets the long factor; the strided passes get M1
     uint64_t M0 = 4096, M1 = M / M0;
+    if(sM1 != 0)
+    {
+        M1 = sM1;
+        M0 = sM0;
+    }
+    else
     {
         // short strided passes make tiny workgroups: keep at least `floor` points in them
         static const char* env   = getenv("ROCFFT_AMD_BLU_M1");

@@ -334,6 +334,35 @@ def test_bluestein_two_level_matches_direct_bins(emu):
         assert abs(y[0, k] - orc.dft_bin(x[0], k)) / np.abs(y).max() < 1e-14
 
 
+def test_bluestein_takes_a_shorter_convolution_length(emu):
+    """Any length >= 2n-1 serves as the convolution length; when one made of compiled kernels is
+    at least 30 % shorter than the next power of two the plan uses it: in one kernel (521 ->
+    1053 instead of 2048), in the three-kernel form (8209 -> 8 x 2057 instead of 32768) and in a
+    strided dimension (2053 -> 64 x 65 instead of 8192).  A length just below a power of two
+    keeps the power of two (1000003 -> 2^21, 1553 -> 4096)."""
+    def lengths_in(text):
+        return [int(v) for v in re.findall(r" n=(\d+) ", text)]
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [521], 8)
+    assert st == 0 and len(passes(text)) == 1 and 1041 <= lengths_in(text)[0] < 1434, text
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [8209], 8)
+    n = lengths_in(text)
+    assert st == 0 and len(n) == 3 and n[0] == n[2] and 16417 <= n[0] * n[1] < 22937, text
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [9, 2053], 2)
+    n = lengths_in(text)
+    assert st == 0 and len(n) == 4 and n[1] >= 64 and 4105 <= n[1] * n[2] < 5734, text
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [1553], 8)
+    assert lengths_in(text) == [4096], text
+    for kind, lengths, batch, prec in [(B.COMPLEX_FORWARD, [131], 3, B.SINGLE), (B.COMPLEX_INVERSE, [521], 3, B.DOUBLE),
+                                       (B.COMPLEX_FORWARD, [2053], 2, B.SINGLE), (B.COMPLEX_FORWARD, [4099], 2, B.SINGLE),
+                                       (B.COMPLEX_INVERSE, [4099], 2, B.DOUBLE), (B.COMPLEX_FORWARD, [8209], 2, B.SINGLE),
+                                       (B.COMPLEX_FORWARD, [8209], 1, B.DOUBLE), (B.COMPLEX_FORWARD, [9, 2053], 2, B.SINGLE),
+                                       (B.COMPLEX_INVERSE, [9, 2053], 1, B.DOUBLE), (B.REAL_FORWARD, [4099], 2, B.SINGLE),
+                                       (B.REAL_INVERSE, [4099], 2, B.DOUBLE), (B.REAL_FORWARD, [1042], 2, B.DOUBLE),
+                                       (B.REAL_INVERSE, [16418], 1, B.SINGLE), (B.COMPLEX_FORWARD, [20011], 1, B.SINGLE)]:
+        H.check(emu, HOST, kind, lengths, batch, prec)
+        H.check(emu, HOST, kind, lengths, batch, prec, inplace=True, scale=0.5)
+
+
 def test_strides_offsets_planar_scale(emu):
     K = B
     # strided + offset 1D
