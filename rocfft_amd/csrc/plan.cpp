@@ -1421,8 +1421,12 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
                 if(!fast_kernel_exists(m0, esize) || !single_kernel_length(m0, esize))
                     continue;
                 uint64_t m1 = std::max<uint64_t>(lo1, (need + m0 - 1) / m0);
-                while(m1 * m0 < lim && !(fast_kernel_exists(m1, esize) && column_kernel_length(m1, esize)))
+                for(int step = 0; step < 64 && m1 * m0 < lim
+                                  && !(fast_kernel_exists(m1, esize) && column_kernel_length(m1, esize));
+                    ++step)
                     ++m1;
+                if(!(fast_kernel_exists(m1, esize) && column_kernel_length(m1, esize)))
+                    continue;
                 if(m1 * m0 < lim && (best == 0 || m1 * m0 < best))
                 {
                     best = m1 * m0;
@@ -1440,7 +1444,12 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     // (checked before any table is computed: a chirp of 10^8 entries takes a minute)
     if(!one && !wide_one && (ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out))
         fail("odd-length real transforms of this size are not implemented");
-    if(!one && sM1 == 0 && !single_kernel_length(M / 4096, esize))
+    // rows of 4096 points in the three-kernel form, 8192 where that keeps the strided factor
+    // within one kernel
+    uint64_t row_len = 4096;
+    if(!one && sM1 == 0 && !single_kernel_length(M / row_len, esize) && single_kernel_length(8192, esize))
+        row_len = 8192;
+    if(!one && sM1 == 0 && !single_kernel_length(M / row_len, esize))
         fail("Bluestein length too large");
     TablePtr chirp      = chirp_table(N, b.precision, b.dry);
     double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
@@ -1506,7 +1515,7 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
         fail("odd-length real transforms of this size are not implemented");
     // M = M1*M0: rows of length M0 are transformed, multiplied and transformed back by
     // one kernel, so that kernel gets the long factor; the strided passes get M1
-    uint64_t M0 = 4096, M1 = M / M0;
+    uint64_t M0 = row_len, M1 = M / M0;
     if(sM1 != 0)
     {
         M1 = sM1;
