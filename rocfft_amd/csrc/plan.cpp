@@ -160,7 +160,8 @@ static TablePtr cached_table(const std::string& key, int precision, bool dry, Ge
         if(TablePtr t = it->second.lock())
             return t;
     HostTable h;
-    gen(h);
+    if(!dry) // a plan that is only described needs no table contents
+        gen(h);
     TablePtr t       = upload_table(h, precision, dry);
     g_cache[k.str()] = t;
     return t;
