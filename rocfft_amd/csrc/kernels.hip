@@ -37,7 +37,10 @@ __device__ __forceinline__ void run_passes(const fftk_params&         p,
             FFTK_CASE(9)
             FFTK_CASE(10)
             FFTK_CASE(11)
+            FFTK_CASE(12)
             FFTK_CASE(13)
+            FFTK_CASE(14)
+            FFTK_CASE(15)
             FFTK_CASE(16)
             FFTK_CASE(17)
 #undef FFTK_CASE

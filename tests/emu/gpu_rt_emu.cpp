@@ -50,7 +50,10 @@ void emu_passes(const fftk_params& p, typename cplx_of<T>::type* lds)
                     EMU_CASE(9)
                     EMU_CASE(10)
                     EMU_CASE(11)
+                    EMU_CASE(12)
                     EMU_CASE(13)
+                    EMU_CASE(14)
+                    EMU_CASE(15)
                     EMU_CASE(16)
                     EMU_CASE(17)
 #undef EMU_CASE

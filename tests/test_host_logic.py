@@ -234,7 +234,7 @@ def test_compiled_schedule_list_is_consistent(emu):
     assert len(rows) == len({r[0] for r in rows}) and len(rows) > 200
     for n, radix, tf, td in rows:
         assert int(np.prod(radix)) == n and 1 <= len(radix) <= 4
-        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 13, 16, 17) for r in radix)
+        assert all(r in (2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17) for r in radix)
         need = max(-(-(n // r) // (17 // r)) for r in radix)
         for t in (tf, td):
             assert t == 0 or need <= t <= 1024
@@ -245,9 +245,10 @@ def test_compiled_schedule_list_is_consistent(emu):
 
 
 # the emulation runs the generic kernel on the schedules of the compiled kernels, composite
-# radices 6, 9 and 10 and the prime radix 17 included
+# radices 6, 9, 10, 12, 14 and 15 and the prime radix 17 included
 @pytest.mark.parametrize("n", [6, 9, 10, 12, 18, 36, 60, 81, 90, 100, 120, 125, 243, 250, 360, 480, 729,
-                               1000, 1536, 2187, 3000, 3645, 4000, 4032, 17, 34, 289, 1156, 2040, 4046, 4080])
+                               1000, 1536, 2187, 3000, 3645, 4000, 4032, 17, 34, 289, 1156, 2040, 4046, 4080,
+                               1728, 2925, 3360, 2002])
 def test_compiled_schedules_on_the_generic_kernel(emu, n):
     H.check(emu, HOST, B.COMPLEX_FORWARD, [n], 3, B.SINGLE)
     H.check(emu, HOST, B.COMPLEX_INVERSE, [n], 2, B.DOUBLE, inplace=True)
