@@ -58,6 +58,27 @@ ROCFFT_EXPORT rocfft_status rocfft_amd_execute_profile(const rocfft_plan     pla
                                                        float*                pass_ms,
                                                        size_t                capacity);
 
+/*
+ * rocfft_execute for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  The plan's work area is a device-resident
+ * array of ROCFFT_AMD_STATIC_WORK_BYTES that the library holds on every GPU it
+ * runs on until the process ends; a work buffer set in `info` is ignored, its
+ * stream is used.  The call allocates and frees nothing.  Plans that need a
+ * larger work area return rocfft_status_invalid_work_buffer (query the need
+ * with rocfft_plan_get_work_buffer_size); load/store callbacks and half
+ * precision, which stage through per-call buffers, return
+ * rocfft_status_failure.  All calls on one GPU share the one array: calls that
+ * overlap in time on the same GPU (different streams or threads) race.
+ * Nothing in the array has to be cleared between calls (every pass writes the
+ * part of the work area it later reads).
+ */
+#define ROCFFT_AMD_STATIC_WORK_BYTES ((size_t)64 << 20)
+ROCFFT_EXPORT rocfft_status rocfft_amd_execute_static(const rocfft_plan     plan,
+                                                      void*                 in_buffer[],
+                                                      void*                 out_buffer[],
+                                                      rocfft_execution_info info);
+
 #ifdef __cplusplus
 }
 #endif

@@ -90,7 +90,11 @@ _PROTOTYPES = {
                                       ctypes.POINTER(ctypes.c_double)],
     "rocfft_amd_execute_profile": [ctypes.c_void_p, _c_void_pp, _c_void_pp, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_float), ctypes.c_size_t],
+    "rocfft_amd_execute_static": [ctypes.c_void_p, _c_void_pp, _c_void_pp, ctypes.c_void_p],
 }
+
+# size of the device-resident work area behind rocfft_amd_execute_static
+STATIC_WORK_BYTES = 64 << 20
 
 EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
 
@@ -279,6 +283,17 @@ class Plan:
 
     def execute(self, in_ptrs, out_ptrs=None, info=None):
         self.lib.check(self.execute_status(in_ptrs, out_ptrs, info), "rocfft_execute")
+
+    def execute_static_status(self, in_ptrs, out_ptrs=None, info=None):
+        """rocfft_amd_execute_static: the work area is the library's own static device array"""
+        ins = (ctypes.c_void_p * 2)(*(list(in_ptrs) + [None])[:2])
+        outs = None
+        if out_ptrs is not None:
+            outs = (ctypes.c_void_p * 2)(*(list(out_ptrs) + [None])[:2])
+        return self.lib.c.rocfft_amd_execute_static(self.handle, ins, outs, info.handle if info else None)
+
+    def execute_static(self, in_ptrs, out_ptrs=None, info=None):
+        self.lib.check(self.execute_static_status(in_ptrs, out_ptrs, info), "rocfft_amd_execute_static")
 
     def passes(self):
         """[(name, bytes read + written)] of the plan's kernel launches, in order"""

@@ -436,8 +436,10 @@ rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement plac
     }
 }
 
+// static_work: take the work area from the library's device-resident array instead of the
+// caller's buffer or a fresh allocation, and refuse whatever would need an allocation
 static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
-                                  rocfft_execution_info info, float* pass_ms)
+                                  rocfft_execution_info info, float* pass_ms, bool static_work = false)
 {
     if(!plan || !in_buffer || !in_buffer[0])
         return rocfft_status_failure;
@@ -468,7 +470,21 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         size_t need   = ep.work_bytes();
         void*  work   = nullptr;
         bool   own    = false;
-        if(need)
+        if(need && static_work)
+        {
+            size_t have = 0;
+            if(fftrt_static_scratch(&work, &have) != 0)
+                return rocfft_status_failure;
+            if(need > have)
+            {
+                fprintf(stderr,
+                        "rocfft_amd_execute_static: the plan needs %zu bytes of work area, the static area "
+                        "holds %zu\n",
+                        need, have);
+                return rocfft_status_invalid_work_buffer;
+            }
+        }
+        else if(need)
         {
             if(info && info->workBuffer)
             {
@@ -501,6 +517,8 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         const bool have_cb   = info && (info->load_cb || info->store_cb);
         const bool half_io   = plan->half_io;
         const bool staging   = have_cb || half_io;
+        if(staging && static_work)
+            return rocfft_status_failure; // staged copies are allocated per call
         auto       cleanup   = [&]() {
             if(own || staging)
                 fftrt_stream_sync(stream);
@@ -644,6 +662,12 @@ rocfft_status rocfft_amd_execute_profile(const rocfft_plan plan, void* in_buffer
     if(!plan || !pass_ms || capacity < plan->exec.passes.size())
         return rocfft_status_invalid_arg_value;
     return execute_impl(plan, in_buffer, out_buffer, info, pass_ms);
+}
+
+rocfft_status rocfft_amd_execute_static(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
+                                        rocfft_execution_info info)
+{
+    return execute_impl(plan, in_buffer, out_buffer, info, nullptr, true);
 }
 
 rocfft_status rocfft_amd_plan_get_pass_count(const rocfft_plan plan, size_t* count)

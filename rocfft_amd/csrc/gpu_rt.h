@@ -67,6 +67,12 @@ int fftrt_launch_fast2d_real(const struct fftk_params* p, int precision, int inv
 int fftrt_has_big32k(void);
 int fftrt_launch_big32k(const struct fftk_big_params* p, void* stream);
 
+// Device-resident work area that exists for the life of the process (one copy per
+// device): its address on the current device and its size.  Used by the execute
+// variant that may not allocate.  Calls that use it at the same time on one device race.
+#define FFTRT_STATIC_SCRATCH_BYTES (64u << 20)
+int fftrt_static_scratch(void** ptr, size_t* bytes);
+
 // event timing, used by the optional per-pass profile log
 int fftrt_event_create(void** ev);
 int fftrt_event_destroy(void* ev);

@@ -308,6 +308,42 @@ int fftrt_launch_real_pre(const struct fftk_real_params* p, int precision, void*
     return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Work area of the execute variant that allocates nothing: a file-scope device
+// array.  Every device holds its own copy at its own address, so the address is
+// looked up once per device (with that device current) and kept; host code never
+// passes the array's name to a kernel or a copy, only the looked-up pointer.
+static __device__ __align__(256) unsigned char scratch[FFTRT_STATIC_SCRATCH_BYTES];
+
+int fftrt_static_scratch(void** ptr, size_t* bytes)
+{
+    constexpr int     MAX_DEVICES = 64;
+    static std::mutex lock;
+    static void*      dev_ptr[MAX_DEVICES]; // zero-initialised: not looked up yet
+    *ptr   = nullptr;
+    *bytes = 0;
+    int dev = 0;
+    int rc  = (int)hipGetDevice(&dev);
+    if(rc)
+        return rc;
+    if(dev < 0 || dev >= MAX_DEVICES)
+        return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if(!dev_ptr[dev])
+    {
+        void* p = nullptr;
+        rc      = (int)hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if(rc)
+            return rc;
+        if(!p)
+            return (int)hipErrorInvalidSymbol;
+        dev_ptr[dev] = p;
+    }
+    *ptr   = dev_ptr[dev];
+    *bytes = FFTRT_STATIC_SCRATCH_BYTES;
+    return 0;
+}
+
 int fftrt_event_create(void** ev)
 {
     return (int)hipEventCreate((hipEvent_t*)ev);

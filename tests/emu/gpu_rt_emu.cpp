@@ -278,6 +278,13 @@ int fftrt_launch_big32k(const struct fftk_big_params*, void*)
     return 1;
 }
 
+int fftrt_static_scratch(void** ptr, size_t* bytes)
+{
+    static std::vector<unsigned char> area(FFTRT_STATIC_SCRATCH_BYTES);
+    *ptr   = area.data();
+    *bytes = area.size();
+    return 0;
+}
 int fftrt_event_create(void** ev)
 {
     *ev = nullptr;
