@@ -11,10 +11,14 @@ Prints ONE JSON line.  `value` is GFLOP/s in the 5*N*log2(N) convention summed
 over the transforms of a step.  `roofline` prices the slowest kernel of the step
 against the HBM peak using per-kernel durations taken with HIP events inside this
 script; `cpu_baseline` times the CPU checker (a port of the algorithm, OpenMP
-across the batch) on a bounded sample of the same workload.  `all_configs` adds
-one short measurement for each of the five benchmark configurations, next to
-torch.fft on the same device (on ROCm that is the reference rocFFT behind
-hipFFT), as reported baselines.
+across the batch) on a bounded sample of the same workload; `cpu_other` adds what
+else the host offers (FFTW or MKL when a dlopen finds them, scipy's pocketfft).
+`all_configs` adds one short measurement for each of the five benchmark
+configurations next to reference rocFFT, timed through the identical harness (the
+same rocfft.h calls on the same buffers, preallocated outputs, caller-owned work
+buffer, same warm-up and step count) in a child process per copy of librocfft
+found on the box; the torch.fft figure (the same library behind hipFFT, with
+PyTorch's allocations inside the timed region) stays as a second column.
 """
 import argparse
 import json
@@ -70,7 +74,7 @@ def workloads():
 class Step:
     """plans, device buffers and execution infos of one workload; run() enqueues one step"""
 
-    def __init__(self, cfg_id, wl, torch, stream_ptr):
+    def __init__(self, cfg_id, wl, torch, stream_ptr, lib=None):
         import inputs
         import rocfft_amd as rf
 
@@ -82,7 +86,7 @@ class Step:
         self.keep = []
         cur = self.x
         for (kind, lengths, batch, prec, inplace) in wl["transforms"]:
-            plan = rf.Plan(rf.INPLACE if inplace else rf.NOTINPLACE, kind, prec, lengths, batch)
+            plan = rf.Plan(rf.INPLACE if inplace else rf.NOTINPLACE, kind, prec, lengths, batch, lib=lib)
             rt = torch.float32 if prec == rf.SINGLE else torch.float64
             ct = torch.complex64 if prec == rf.SINGLE else torch.complex128
             total = 1
@@ -97,7 +101,7 @@ class Step:
                 out = torch.empty((batch, total), dtype=rt, device=dev)
             else:
                 out = torch.empty((batch, total), dtype=ct, device=dev)
-            info = rf.ExecutionInfo()
+            info = rf.ExecutionInfo(lib)
             info.set_stream(stream_ptr)
             wb = plan.work_buffer_size
             if wb:
@@ -185,8 +189,9 @@ def cpu_baseline(cfg_id, wl, budget_s=12.0):
                 % (nb, full_batch, "x".join(map(str, lengths)), t, threads))
 
 
-def reference_rocfft_ms(torch, cfg_id, step, reps=5):
-    """torch.fft on the same device buffers (reference rocFFT behind hipFFT); median ms per step"""
+def torch_fft_ms(torch, cfg_id, step, reps=5):
+    """torch.fft on the same input (reference rocFFT behind hipFFT, PyTorch's output
+    allocations inside the timed region); median ms per step"""
     x = step.x
 
     def run():
@@ -218,6 +223,168 @@ def reference_rocfft_ms(torch, cfg_id, step, reps=5):
         return None
 
 
+def reference_library_paths():
+    """copies of the reference library on this machine: the system ROCm's and the one PyTorch bundles"""
+    import importlib.util
+
+    paths = []
+    for p in ("/opt/rocm/lib/librocfft.so.0",):
+        if os.path.exists(p):
+            paths.append(p)
+    spec = importlib.util.find_spec("torch")
+    if spec and spec.origin:
+        p = os.path.join(os.path.dirname(spec.origin), "lib", "librocfft.so")
+        if os.path.exists(p):
+            paths.append(p)
+    return paths
+
+
+def reference_child(path, warmup, steps):
+    """(child process) the five configurations on the library at `path` through the same Step
+    harness as this library; prints one JSON line {"version": ..., "ms": {name: ms}}"""
+    import torch
+
+    import rocfft_amd.binding as B
+
+    lib = B.Library(path, extensions=False)
+    lib.setup()
+    out = {"path": path, "version": lib.version(), "ms": {}, "steps": steps, "warmup": warmup}
+    stream_ptr = torch.cuda.current_stream().cuda_stream
+    wls = workloads()
+    for cid in sorted(wls):
+        try:
+            step = Step(cid, wls[cid], torch, stream_ptr, lib=lib)
+            ms, _ = time_steps(torch, step, warmup, steps)
+            out["ms"][wls[cid]["name"]] = ms
+            del step
+            torch.cuda.empty_cache()
+        except Exception as e:  # noqa: BLE001
+            out["ms"][wls[cid]["name"]] = None
+            out.setdefault("errors", {})[wls[cid]["name"]] = repr(e)[:200]
+    print(json.dumps(out))
+
+
+def reference_rocfft(warmup, steps, timeout_s=240):
+    """runs reference_child once per copy of the reference library, each in its own process
+    (a library that cannot share this process's HIP runtime must not take the benchmark down)"""
+    import subprocess
+
+    results = []
+    for path in reference_library_paths():
+        rec = {"path": path, "version": None, "ms": {}}
+        try:
+            p = subprocess.run([sys.executable, os.path.abspath(__file__), "--reference-lib", path, "--steps",
+                                str(steps), "--warmup", str(warmup)], capture_output=True, text=True,
+                               timeout=timeout_s)
+            line = [ln for ln in p.stdout.strip().splitlines() if ln.startswith("{")]
+            if p.returncode == 0 and line:
+                rec = json.loads(line[-1])
+            else:
+                rec["error"] = ("exit %d: " % p.returncode) + p.stderr.strip()[-200:]
+        except Exception as e:  # noqa: BLE001
+            rec["error"] = repr(e)[:200]
+        results.append(rec)
+    return results
+
+
+def cpu_other(cfg_id, wl, budget_s=6.0):
+    """what else the host offers for the same workload: the reference's CPU path is FFTW
+    (clients/tests/CMakeLists.txt:128-129), looked for with dlopen together with MKL's FFTW
+    interface; scipy's pocketfft (threads stated) is timed in any case.  Configuration 2 only."""
+    import ctypes
+
+    import numpy as np
+
+    found = {}
+    for name in ("libfftw3f.so.3", "libfftw3.so.3", "libfftw3f_threads.so.3", "libfftw3f_omp.so.3", "libmkl_rt.so",
+                 "libmkl_rt.so.2"):
+        try:
+            ctypes.CDLL(name)
+            found[name] = True
+        except OSError:
+            found[name] = False
+    out = {"dlopen": found}
+    if cfg_id != 2:
+        return out
+    import inputs
+
+    n, full = 65536, 4096
+    threads = min(16, os.cpu_count() or 1)
+    nb = 256
+    x = inputs.config_input(2, 0, nb).astype(np.float32)
+    try:
+        import scipy.fft as sf
+
+        def run():
+            return sf.irfft(sf.rfft(x, axis=1, workers=threads), n=n, axis=1, workers=threads)
+
+        run()
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < budget_s and reps < 20:
+            run()
+            reps += 1
+        t = (time.perf_counter() - t0) / reps
+        out["pocketfft"] = dict(value=wl["flops"] * (nb / full) / t / 1e9, unit="GFLOP/s", cores=threads,
+                                kind="scipy.fft (pocketfft) float32, rfft + irfft",
+                                sample="%d of %d transforms of %d, %.2f s per repetition, %d workers"
+                                % (nb, full, n, t, threads))
+    except Exception as e:  # noqa: BLE001
+        out["pocketfft"] = {"error": repr(e)[:200]}
+    if found.get("libfftw3f.so.3"):
+        try:
+            out["fftw"] = fftw_r2c_c2r(x, n, nb, wl, full, budget_s)
+        except Exception as e:  # noqa: BLE001
+            out["fftw"] = {"error": repr(e)[:200]}
+    else:
+        out["fftw"] = None  # not installed on this machine
+    return out
+
+
+def fftw_r2c_c2r(x, n, nb, wl, full, budget_s):
+    """FFTW single precision, batched contiguous out-of-place plans with FFTW_ESTIMATE as the
+    reference's tests make them (shared/rocfft_against_fftw.h:108-142); one thread unless the
+    threads library is present"""
+    import ctypes
+
+    import numpy as np
+
+    fw = ctypes.CDLL("libfftw3f.so.3")
+    threads = 1
+    for tl in ("libfftw3f_omp.so.3", "libfftw3f_threads.so.3"):
+        try:
+            ft = ctypes.CDLL(tl, mode=ctypes.RTLD_GLOBAL)
+            ft.fftwf_init_threads()
+            threads = min(16, os.cpu_count() or 1)
+            ft.fftwf_plan_with_nthreads(threads)
+            break
+        except (OSError, AttributeError):
+            continue
+    h = n // 2 + 1
+    y = np.empty((nb, h), dtype=np.complex64)
+    z = np.empty((nb, n), dtype=np.float32)
+    nn = (ctypes.c_int * 1)(n)
+    fw.fftwf_plan_many_dft_r2c.restype = ctypes.c_void_p
+    fw.fftwf_plan_many_dft_c2r.restype = ctypes.c_void_p
+    FFTW_ESTIMATE = 1 << 6
+    pf = fw.fftwf_plan_many_dft_r2c(1, nn, nb, ctypes.c_void_p(x.ctypes.data), None, 1, n,
+                                    ctypes.c_void_p(y.ctypes.data), None, 1, h, FFTW_ESTIMATE)
+    pb = fw.fftwf_plan_many_dft_c2r(1, nn, nb, ctypes.c_void_p(y.ctypes.data), None, 1, h,
+                                    ctypes.c_void_p(z.ctypes.data), None, 1, n, FFTW_ESTIMATE)
+    if not pf or not pb:
+        raise RuntimeError("fftwf_plan_many_dft failed")
+    fw.fftwf_execute.argtypes = [ctypes.c_void_p]
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < budget_s and reps < 20:
+        fw.fftwf_execute(pf)
+        fw.fftwf_execute(pb)
+        reps += 1
+    t = (time.perf_counter() - t0) / reps
+    return dict(value=wl["flops"] * (nb / full) / t / 1e9, unit="GFLOP/s", cores=threads, kind="FFTW 3 float32",
+                sample="%d of %d transforms of %d, %.2f s per repetition" % (nb, full, n, t))
+
+
 def measure_config(torch, cfg_id, wl, stream_ptr, warmup, steps, prof_reps):
     step = Step(cfg_id, wl, torch, stream_ptr)
     ms, dev_ms = time_steps(torch, step, warmup, steps)
@@ -232,6 +399,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (default 2)")
     ap.add_argument("--no-extras", action="store_true", help="skip all_configs and the CPU baseline")
+    ap.add_argument("--reference-lib", default=None,
+                    help="(used by this script for its child processes) time the five configurations on the "
+                         "rocfft.h library at this path and print them as JSON")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB) ten times: "
                          "the known-size kernel the rocprofv3 FETCH_SIZE/WRITE_SIZE counters are scaled by")
@@ -242,6 +412,12 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    # the reference library's figures come from child processes, started before this process
+    # initialises the GPU
+    refs = []
+    if not (args.no_extras or args.reference_lib or args.calibrate_copy):
+        refs = reference_rocfft(2, 10)
+
     import torch
 
     import rocfft_amd as rf
@@ -249,6 +425,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU", file=sys.stderr)
         sys.exit(1)
+    if args.reference_lib:
+        reference_child(args.reference_lib, args.warmup, args.steps)
+        return
     if args.calibrate_copy:
         n = 1 << 28  # float32 elements = 1 GiB
         src = torch.rand(n, dtype=torch.float32, device="cuda:0")
@@ -299,31 +478,39 @@ def main():
                     for n, b, t in prof],
     }
     if not args.no_extras:
-        ref_ms = reference_rocfft_ms(torch, args.config, step)
+        tf_ms = torch_fft_ms(torch, args.config, step)
         allc = {}
         for cid in sorted(wls):
             if cid == args.config:
                 s2, m2, p2 = step, ms, prof
-                r2 = ref_ms
+                t2 = tf_ms
             else:
                 del step
                 torch.cuda.empty_cache()
                 s2, m2, _, p2 = measure_config(torch, cid, wls[cid], stream_ptr, 2, 10, 2)
-                r2 = reference_rocfft_ms(torch, cid, s2)
+                t2 = torch_fft_ms(torch, cid, s2)
                 step = s2
             w2 = wls[cid]
+            # reference rocFFT through the identical harness: the fastest copy found on this machine
+            same = [(r["ms"].get(w2["name"]), r.get("version"), r.get("path")) for r in refs
+                    if r.get("ms", {}).get(w2["name"])]
+            r2 = min(same) if same else (None, None, None)
             allc[w2["name"]] = {
                 "ms": m2, "GFLOPs": w2["flops"] / (m2 * 1e-3) / 1e9,
                 "GBps": w2["bytes"] / (m2 * 1e-3) / 1e9,
                 "hbm_frac": w2["bytes"] / (m2 * 1e-3) / 1e9 / HBM_PEAK_GBS,
                 "kernels": len(p2),
-                "reference_rocfft_ms": r2,
-                "reference_rocfft_GFLOPs": (w2["flops"] / (r2 * 1e-3) / 1e9) if r2 else None,
+                "reference_rocfft_ms": r2[0],
+                "reference_rocfft_version": r2[1],
+                "reference_rocfft_GFLOPs": (w2["flops"] / (r2[0] * 1e-3) / 1e9) if r2[0] else None,
+                "torch_fft_ms": t2,
             }
         out["all_configs"] = allc
+        out["reference_rocfft"] = refs
         del step
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline(args.config, wl)
+        out["cpu_other"] = cpu_other(args.config, wl)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

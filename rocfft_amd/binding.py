@@ -102,13 +102,17 @@ EXPORTED_SYMBOLS = tuple(_PROTOTYPES)
 class Library:
     """One loaded copy of the shared library."""
 
-    def __init__(self, path=None):
+    def __init__(self, path=None, extensions=True):
+        """extensions=False loads any library that speaks rocfft.h (the reference's own
+        librocfft.so, to time it through the same calls): the rocfft_amd_* entry points are
+        then not looked up."""
         path = path or library_path()
         if not os.path.exists(path):
             raise FileNotFoundError(
                 "%s is missing: build it with __graft_entry__.build() (hipcc, gfx950); "
                 "there is no fallback implementation" % path)
         self.path = path
+        self.extensions = extensions
         # PyTorch wheels carry their own copy of the HIP runtime under the same soname.
         # When a process uses both, torch must be loaded first so that this library
         # binds to the runtime torch initialises (one runtime per process).
@@ -118,6 +122,8 @@ class Library:
             pass
         self.c = ctypes.CDLL(path)
         for name, args in _PROTOTYPES.items():
+            if not extensions and name.startswith("rocfft_amd_"):
+                continue
             fn = getattr(self.c, name)
             fn.argtypes = args
             fn.restype = ctypes.c_int

@@ -60,6 +60,7 @@ struct fftk_params
     uint32_t nthreads;
     uint32_t grid;       // number of workgroups
     uint32_t xcd_remap;  // renumber workgroups so that each XCD gets a contiguous range of tiles
+    uint32_t oc0_first;  // outer axis 0 runs faster than the tile index in the workgroup numbering
     uint32_t fast;       // 1 = a kernel with this exact pass schedule is compiled in: use it
     uint32_t direct_in;  // fast kernel: first pass loads global memory straight into registers
     uint32_t direct_out; // fast kernel: last pass stores straight from registers

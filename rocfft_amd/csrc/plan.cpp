@@ -33,6 +33,7 @@ static const size_t   COL_RUN_BYTES  = 128;
 static const bool g_use_fast = !getenv("ROCFFT_AMD_GENERIC");
 // ROCFFT_AMD_NO_XCD_REMAP=1 keeps the hardware's round-robin workgroup order (A/B comparisons)
 static const bool g_xcd_remap = !getenv("ROCFFT_AMD_NO_XCD_REMAP");
+static const bool g_share_first = !getenv("ROCFFT_AMD_NO_SHARE_FIRST");
 
 struct PlanError : std::runtime_error
 {
@@ -705,6 +706,15 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         k.oc[i]   = 1;
         k.o_is[i] = k.o_os[i] = 0;
     }
+    // A pass that multiplies by a long table (chirp, chirp spectrum) indexes it with the tile or
+    // an outer axis; the remaining plain axis (the signals of a batch) re-reads the same entries.
+    // That axis goes first in the workgroup numbering, so that the re-reads follow one another.
+    // (Tables beyond a megabyte only: shorter ones stay in L2 anyway.  One outer axis only: with
+    // more, neighbouring column tiles would no longer be neighbours in the numbering.)
+    bool         shared_table_axis = false;
+    const size_t table_bytes       = std::max(s.chirp ? s.chirp->bytes : 0, s.convb ? s.convb->bytes : 0);
+    if(table_bytes >= (1u << 20) && ax.size() == 1 && !ax[0].aux && ax[0].cnt > 1)
+        shared_table_axis = true;
     for(size_t i = 0; i < ax.size(); ++i)
     {
         k.oc[i]   = ax[i].cnt;
@@ -783,6 +793,11 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         const int64_t line  = 128 / (precision ? 8 : 4); // scalars per 128 bytes
         const bool    split = (k.in_fast_tile && (k.t_is % line)) || (k.out_fast_tile && (k.t_os % line));
         k.xcd_remap         = (g_xcd_remap && column && split && rec.grid >= 64) ? 1 : 0;
+    }
+    if(shared_table_axis && g_share_first)
+    {
+        k.oc0_first = 1;
+        k.xcd_remap = (g_xcd_remap && rec.grid >= 64) ? 1 : 0;
     }
 
     k.flags    = s.flags;
@@ -2735,6 +2750,10 @@ std::string ExecPlan::describe() const
               << " load " << k.load_op << " store " << k.store_op << (r.vec_ok ? " vec" : " scalar");
             if(r.lean_ok)
                 o << " lean";
+            if(k.xcd_remap)
+                o << " xcd_ranges";
+            if(k.oc0_first)
+                o << " batch_first";
             if(k.fast)
                 o << " fast" << (k.direct_in ? " direct_in" : " staged_in")
                   << (k.direct_out ? " direct_out" : " staged_out") << (k.stage_io ? " tile_copy" : "");

@@ -43,10 +43,23 @@ FFT_DEV void tile_decode(const fftk_params& p, uint32_t bid, TileCtx<T>& c)
         bid = xcd * qd + (xcd < rm ? xcd : rm) + idx;
     }
     uint32_t ntile = (p.tile_cnt + p.W - 1) >> p.wshift;
-    uint32_t tb    = bid % ntile;
-    bid /= ntile;
-    c.oi[0] = bid % p.oc[0];
-    bid /= p.oc[0];
+    uint32_t tb;
+    if(p.oc0_first)
+    {
+        // workgroups that differ in outer index 0 only (the signals of a batch) are neighbours:
+        // they read the same rows of a chirp or spectrum table, one after the other in one L2
+        c.oi[0] = bid % p.oc[0];
+        bid /= p.oc[0];
+        tb = bid % ntile;
+        bid /= ntile;
+    }
+    else
+    {
+        tb = bid % ntile;
+        bid /= ntile;
+        c.oi[0] = bid % p.oc[0];
+        bid /= p.oc[0];
+    }
     c.oi[1] = bid % p.oc[1];
     c.oi[2] = bid / p.oc[1];
     c.tile0 = tb << p.wshift;
