@@ -467,7 +467,11 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         if((planar(pr.in_type) && !in[1]) || (planar(pr.out_type) && !out[1]))
             return rocfft_status_failure;
         void*  stream = info ? info->stream : nullptr;
-        size_t need   = ep.work_bytes();
+        // the work area of the pass list these buffers get (staged copies are aligned allocations)
+        const bool staged_run = plan->half_io || (info && (info->load_cb || info->store_cb));
+        size_t     need       = staged_run ? ep.own_work_bytes()
+                                           : select_exec_plan(ep, in, out, info ? info->workBuffer : nullptr)
+                                           .own_work_bytes();
         void*  work   = nullptr;
         bool   own    = false;
         if(need && static_work)

@@ -136,7 +136,6 @@ struct Fast2dRealShape
 template <typename CfgA, typename Sh>
 struct FkRealRowAddr
 {
-    template <int X, int ELEM_BYTES>
     static FFT_DEV uint32_t at(uint32_t row, uint32_t j)
     {
         return Sh::at(row, j);
@@ -316,7 +315,7 @@ __device__ __forceinline__ void fast2d_c2r_body(const fftk_params& p, typename c
 #pragma unroll
                 for(int kk = 0; kk < RL; ++kk)
                     if(fk_live<CfgB, LAST>(tt, s))
-                        lds[Col::template at<-1, 8>(base, tt + s * CfgB::TPT + kk * CL)] = c_swap(r[s * RL + kk]);
+                        lds[Col::at(base, tt + s * CfgB::TPT + kk * CL)] = c_swap(r[s * RL + kk]);
         }
     }
     __syncthreads();

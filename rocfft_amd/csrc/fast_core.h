@@ -80,23 +80,6 @@ FFT_DEV uint32_t fk_addr(uint32_t w, uint32_t j)
     return w * Cfg::PITCH + j + (j >> Cfg::PADSHIFT);
 }
 
-// LDS position of element j during exchange X (between pass X and pass X + 1).  Every exchange
-// rewrites the whole transform, so each may pad in its own way.  The default (one pad element
-// per 16) keeps the strided writes of a pass apart but lets lanes 0 and 31 of the unit-stride
-// reads that follow meet in one bank pair: 8-byte elements are served 32 lanes at a time from
-// 32 bank pairs, and j + (j >> 4) puts lane 31 on pair 0 again -- every such read takes two
-// turns.  Schedules that open with two radix-16 passes have a padding that serves all four
-// access patterns in one turn: one pad per 32 elements for the first exchange (writes 16 apart),
-// two per 32 for the later ones (writes of lanes 16 apart land 256 elements apart).
-template <typename Cfg, int X, int ELEM_BYTES>
-FFT_DEV uint32_t fk_xaddr(uint32_t w, uint32_t j)
-{
-    if constexpr(ELEM_BYTES == 8 && Cfg::R0 == 16 && Cfg::R1 == 16 && Cfg::N >= 1024 && Cfg::TPT >= 32 && X >= 0)
-        return w * Cfg::PITCH + j + (X == 0 ? (j >> 5) : 2 * (j >> 5));
-    else
-        return fk_addr<Cfg>(w, j);
-}
-
 // does lane tt have a butterfly in slot s of pass P?
 template <typename Cfg, int P>
 FFT_DEV bool fk_live(uint32_t tt, int s)
@@ -124,21 +107,17 @@ FFT_DEV uint32_t fk_out_pos(uint32_t tt, int s, int k)
 // Where element j of the transform that the handle `w` names lives in LDS.  Rows of a tile:
 // w is the transform's index in the tile.  FkStrideAddr: w is the LDS index of element 0 and
 // the elements are STRIDE apart (the columns of a 2D tile held row by row).
-// X names the exchange the access belongs to (-1: not an exchange between two passes: the
-// staged input or output of the tile, which tile_load / tile_store address in the default way).
 template <typename Cfg>
 struct FkRowAddr
 {
-    template <int X, int ELEM_BYTES>
     static FFT_DEV uint32_t at(uint32_t w, uint32_t j)
     {
-        return fk_xaddr<Cfg, X, ELEM_BYTES>(w, j);
+        return fk_addr<Cfg>(w, j);
     }
 };
 template <int STRIDE>
 struct FkStrideAddr
 {
-    template <int X, int ELEM_BYTES>
     static FFT_DEV uint32_t at(uint32_t base, uint32_t j)
     {
         return base + j * (uint32_t)STRIDE;
@@ -157,7 +136,7 @@ FFT_DEV void fk_read(const typename cplx_of<T>::type* lds, uint32_t w, uint32_t 
         {
 #pragma unroll
             for(int k = 0; k < R; ++k)
-                r[s * R + k] = lds[A::template at<P - 1, (int)sizeof(typename cplx_of<T>::type)>(w, fk_in_pos<Cfg, P>(tt, s, k))];
+                r[s * R + k] = lds[A::at(w, fk_in_pos<Cfg, P>(tt, s, k))];
         }
 }
 
@@ -173,7 +152,7 @@ FFT_DEV void fk_write(typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
         {
 #pragma unroll
             for(int k = 0; k < R; ++k)
-                lds[A::template at<(P < Cfg::NP - 1 ? P : -1), (int)sizeof(typename cplx_of<T>::type)>(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
+                lds[A::at(w, fk_out_pos<Cfg, P>(tt, s, k))] = r[s * R + k];
         }
 }
 

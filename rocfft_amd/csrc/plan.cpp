@@ -30,7 +30,15 @@ static const uint32_t PADSHIFT       = 4;
 static const size_t   COL_RUN_BYTES  = 128;
 
 // ROCFFT_AMD_GENERIC=1 forces the generic tile kernel everywhere (A/B comparisons)
-static const bool g_use_fast = !getenv("ROCFFT_AMD_GENERIC");
+static const bool g_use_fast_env = !getenv("ROCFFT_AMD_GENERIC");
+// set while the alternate plan for buffers without vector alignment is being built: only the
+// run-time-schedule tile kernel, which has a scalar-access form for every pass
+static thread_local bool t_generic_only = false;
+static bool use_fast_kernels()
+{
+    return g_use_fast_env && !t_generic_only;
+}
+#define g_use_fast use_fast_kernels()
 // ROCFFT_AMD_NO_XCD_REMAP=1 keeps the hardware's round-robin workgroup order (A/B comparisons)
 static const bool g_xcd_remap = !getenv("ROCFFT_AMD_NO_XCD_REMAP");
 static const bool g_share_first = !getenv("ROCFFT_AMD_NO_SHARE_FIRST");
@@ -2307,7 +2315,7 @@ static void check_sizes(const Problem& p)
         throw PlanError(rocfft_status_failure, "bad batch");
 }
 
-rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::string& err)
+static rocfft_status build_exec_plan_once(const Problem& p, ExecPlan& plan, bool dry, std::string& err)
 {
     try
     {
@@ -2554,6 +2562,45 @@ rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::s
     }
 }
 
+// true when the pass has no form for buffers aligned to a scalar only
+static bool needs_vector_alignment(const PassRec& r)
+{
+    if(r.kind == PASS_BIG || r.kind == PASS_2D)
+        return true;
+    return r.kind == PASS_TILE && r.kp.fast && r.kp.nthreads > 512;
+}
+
+rocfft_status build_exec_plan(const Problem& p, ExecPlan& plan, bool dry, std::string& err)
+{
+    rocfft_status st = build_exec_plan_once(p, plan, dry, err);
+    if(st != rocfft_status_success)
+        return st;
+    bool any = false;
+    for(const PassRec& r : plan.passes)
+        any = any || needs_vector_alignment(r);
+    if(any)
+    {
+        struct Mode
+        {
+            Mode()
+            {
+                t_generic_only = true;
+            }
+            ~Mode()
+            {
+                t_generic_only = false;
+            }
+        } mode;
+        auto        alt = std::make_shared<ExecPlan>();
+        std::string alt_err;
+        // a transform the tile kernel alone cannot plan keeps the single pass list (and the
+        // executor's refusal of unaligned buffers)
+        if(build_exec_plan_once(p, *alt, dry, alt_err) == rocfft_status_success)
+            plan.unaligned = alt;
+    }
+    return rocfft_status_success;
+}
+
 // ---------------------------------------------------------------------------
 // executor (reference: TransformPowX, library/src/powX.cpp:525-957)
 
@@ -2562,21 +2609,51 @@ static bool aligned(const void* p, size_t a)
     return ((uintptr_t)p % a) == 0;
 }
 
+const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work)
+{
+    if(!plan.unaligned)
+        return plan;
+    const size_t scalar = plan.precision ? 8 : 4;
+    auto         base   = [&](const IoRef& io) -> const char* {
+        switch(io.buf)
+        {
+        case BUF_IN:
+            return static_cast<const char*>(in[0]);
+        case BUF_OUT:
+            return static_cast<const char*>(out[0]);
+        default:
+            // the regions of the work buffer start at multiples of the element size
+            return static_cast<const char*>(work);
+        }
+    };
+    for(const PassRec& rec : plan.passes)
+    {
+        if(!needs_vector_alignment(rec))
+            continue;
+        const size_t need = rec.kind == PASS_BIG ? 8 : plan.elem_bytes;
+        const char*  s0   = base(rec.src);
+        const char*  d0   = base(rec.dst);
+        if((s0 && !aligned(s0 + rec.src.off0 * (int64_t)scalar, need))
+           || (d0 && !aligned(d0 + rec.dst.off0 * (int64_t)scalar, need)))
+            return *plan.unaligned;
+    }
+    return plan;
+}
+
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
                             void* stream, float* pass_ms)
 {
-    // optional per-pass timing (the reference's profile layer does the same with
-    // hipEvents around every kernel, library/src/powX.cpp:817-883)
-    std::vector<void*> events;
-    if(pass_ms)
     {
-        events.resize(plan.passes.size() + 1, nullptr);
-        for(void*& e : events)
-            if(fftrt_event_create(&e) != 0)
-                return rocfft_status_failure;
-        fftrt_event_record(events[0], stream);
+        const ExecPlan& chosen = select_exec_plan(plan, in, out, work);
+        if(&chosen != &plan)
+        {
+            // (per-pass timings describe the primary pass list: not reported for the other one)
+            if(pass_ms)
+                for(size_t i = 0; i < plan.passes.size(); ++i)
+                    pass_ms[i] = -1.0f;
+            return run_exec_plan(chosen, in, out, work, stream, nullptr);
+        }
     }
-    size_t pass_index = 0;
     const size_t scalar = plan.precision ? 8 : 4;
     char*        tmp    = static_cast<char*>(work);
     char*        blu    = tmp ? tmp + plan.tmp_elems * plan.elem_bytes : nullptr;
@@ -2617,6 +2694,28 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             p1 = p0 + io.im_delta * (int64_t)scalar;
         return true;
     };
+    // optional per-pass timing (the reference's profile layer does the same with
+    // hipEvents around every kernel, library/src/powX.cpp:817-883)
+    struct Events
+    {
+        std::vector<void*> v;
+        ~Events()
+        {
+            for(void* e : v)
+                if(e)
+                    fftrt_event_destroy(e);
+        }
+    } ev;
+    std::vector<void*>& events = ev.v;
+    if(pass_ms)
+    {
+        events.resize(plan.passes.size() + 1, nullptr);
+        for(void*& e : events)
+            if(fftrt_event_create(&e) != 0)
+                return rocfft_status_failure;
+        fftrt_event_record(events[0], stream);
+    }
+    size_t pass_index = 0;
     for(const PassRec& rec : plan.passes)
     {
         char *s0, *s1, *d0, *d1;
@@ -2705,8 +2804,6 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
         for(size_t i = 0; i < plan.passes.size(); ++i)
             if(fftrt_event_elapsed_ms(events[i], events[i + 1], &pass_ms[i]) != 0)
                 pass_ms[i] = -1.0f;
-        for(void* e : events)
-            fftrt_event_destroy(e);
     }
     return rocfft_status_success;
 }
@@ -2770,6 +2867,9 @@ std::string ExecPlan::describe() const
               << r.rp.rows2;
         o << "\n";
     }
+    if(unaligned)
+        o << "  for buffers without vector alignment: " << unaligned->passes.size() << " passes, work buffer "
+          << unaligned->own_work_bytes() << " bytes\n";
     return o.str();
 }
 

@@ -12,6 +12,7 @@
 
 #include "kparams.h"
 #include "rocfft/rocfft.h"
+#include <algorithm>
 #include <memory>
 #include <string>
 #include <vector>
@@ -100,9 +101,19 @@ struct ExecPlan
     size_t               cpx_elems  = 0; // complex elements of the real-as-complex scratch
     size_t               elem_bytes = 8; // bytes per complex element
     bool                 inplace    = false;
-    size_t               work_bytes() const
+    // Passes whose kernels move (re, im) pairs with one access and have no scalar-access form
+    // (the one-workgroup 32768-point and small-2D kernels, compiled kernels with more than 512
+    // threads) cannot take buffers that are only aligned to a scalar.  A plan with such passes
+    // carries a second pass list made of run-time-schedule tile passes only, used by the
+    // executor when a buffer fails the alignment test (the reference accepts such buffers).
+    std::shared_ptr<ExecPlan> unaligned;
+    size_t                    own_work_bytes() const
     {
         return (tmp_elems + blu_elems + cpx_elems) * elem_bytes;
+    }
+    size_t work_bytes() const
+    {
+        return unaligned ? std::max(own_work_bytes(), unaligned->own_work_bytes()) : own_work_bytes();
     }
     std::string describe() const;
 };
@@ -117,6 +128,11 @@ rocfft_status build_exec_plan(const Problem& prob, ExecPlan& plan, bool dry_run,
 // milliseconds is written there (the call then waits for the stream).
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
                             void* stream, float* pass_ms = nullptr);
+
+// The pass list run_exec_plan will use for these buffers: the plan itself, or its `unaligned`
+// list when a buffer fails the alignment one of the plan's passes needs.  `work` may be null
+// (not allocated yet: allocations are aligned).
+const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work);
 
 // drops cached tables that no plan uses any more
 void table_cache_clear();

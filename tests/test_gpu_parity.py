@@ -261,6 +261,59 @@ def test_c2r_ignores_imaginary_dc_and_nyquist(gpu):
         assert np.array_equal(y1, y2), n
 
 
+def test_buffers_aligned_to_a_scalar_only(gpu):
+    """Base pointers offset by one scalar.  The kernels that move (re, im) pairs with one
+    access have no form for such buffers; plans that use them carry a second pass list made
+    of the tile kernel alone, which the executor takes.  The reference accepts such buffers
+    (its kernels address scalars)."""
+    lib, be = gpu
+    torch = be.torch
+    cases = [(B.REAL_FORWARD, B.SINGLE, [65536], 3), (B.REAL_INVERSE, B.SINGLE, [65536], 3),
+             (B.COMPLEX_FORWARD, B.SINGLE, [32768], 2), (B.COMPLEX_FORWARD, B.SINGLE, [16384], 3),
+             (B.COMPLEX_INVERSE, B.SINGLE, [32, 32], 5), (B.REAL_FORWARD, B.SINGLE, [16, 16], 7),
+             (B.COMPLEX_FORWARD, B.DOUBLE, [64, 16], 3)]
+    for kind, prec, lengths, batch in cases:
+        rt = torch.float32 if prec == B.SINGLE else torch.float64
+        total = int(np.prod(lengths))
+        herm = total // lengths[0] * (lengths[0] // 2 + 1)
+        n_in = {B.REAL_FORWARD: total, B.REAL_INVERSE: 2 * herm}.get(kind, 2 * total) * batch
+        n_out = {B.REAL_FORWARD: 2 * herm, B.REAL_INVERSE: total}.get(kind, 2 * total) * batch
+        plan = B.Plan(B.NOTINPLACE, kind, prec, lengths, batch, lib=lib)
+        x = (inputs.torch_uniform01(torch, be.dev, 31, 0, n_in) - 0.5).to(rt)
+        if kind == B.REAL_INVERSE:
+            # a Hermitian input: the forward transform of real data
+            fwd = B.Plan(B.NOTINPLACE, B.REAL_FORWARD, prec, lengths, batch, lib=lib)
+            real = (inputs.torch_uniform01(torch, be.dev, 32, 0, total * batch) - 0.5).to(rt)
+            fwd.execute([real.data_ptr()], [x.data_ptr()])
+            torch.cuda.synchronize()
+        want = torch.full((n_out,), float("nan"), dtype=rt, device=be.dev)
+        plan.execute([x.clone().data_ptr()], [want.data_ptr()])
+        torch.cuda.synchronize()
+        # the same data one scalar into larger allocations
+        xin = torch.zeros(n_in + 1, dtype=rt, device=be.dev)
+        xin[1:] = x
+        yout = torch.full((n_out + 2,), 7.0, dtype=rt, device=be.dev)
+        info = B.ExecutionInfo(lib)
+        wb = plan.work_buffer_size
+        if wb:
+            work = torch.empty(wb, dtype=torch.uint8, device=be.dev)
+            info.set_work_buffer(work.data_ptr(), wb)
+        plan.execute([xin[1:].data_ptr()], [yout[1:].data_ptr()], info)
+        torch.cuda.synchronize()
+        assert yout[0].item() == 7.0 and yout[-1].item() == 7.0, (kind, lengths)
+        got = yout[1:-1]
+        assert torch.isfinite(got).all(), (kind, lengths)
+        l2, li = tnorm(torch, got, want)
+        tol = 1e-5 if prec == B.SINGLE else 1e-13
+        assert l2 <= tol and li <= tol, (kind, lengths, l2, li)
+        # and without a caller's work buffer (the library allocates what this pass list needs)
+        yout.fill_(7.0)
+        plan.execute([xin[1:].data_ptr()], [yout[1:].data_ptr()])
+        torch.cuda.synchronize()
+        l2, li = tnorm(torch, yout[1:-1], want)
+        assert l2 <= tol and li <= tol, (kind, lengths, l2, li)
+
+
 def test_work_buffer_contract(gpu):
     lib, be = gpu
     torch = be.torch
