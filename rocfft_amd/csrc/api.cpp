@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <sstream>
 #include <string>
@@ -35,6 +36,35 @@ struct rocfft_plan_description_t
     bool                distributed  = false; // a field or communicator was attached
 };
 
+// Device buffers a plan keeps for executions that stage through copies (load/store callbacks,
+// half precision): the copies of the input and output arrays and, when the caller sets no work
+// buffer, the work area.  One set per stream the plan has been executed on, allocated by the
+// first such execution on that stream and released with the plan, so that later executions
+// allocate nothing, do not wait for the stream and can be captured into a graph.
+struct StageSet
+{
+    void*  in[2]    = {nullptr, nullptr};
+    void*  out[2]   = {nullptr, nullptr};
+    void*  work     = nullptr;
+    size_t in_bytes = 0, out_bytes = 0, work_bytes = 0;
+    bool   shared   = false; // in-place: out[] are in[]
+    void   release()
+    {
+        for(int i = 0; i < 2; ++i)
+        {
+            if(out[i] && !shared)
+                fftrt_free(out[i]);
+            if(in[i])
+                fftrt_free(in[i]);
+            in[i] = out[i] = nullptr;
+        }
+        if(work)
+            fftrt_free(work);
+        work     = nullptr;
+        in_bytes = out_bytes = work_bytes = 0;
+    }
+};
+
 struct rocfft_plan_t
 {
     Problem     prob;
@@ -42,6 +72,15 @@ struct rocfft_plan_t
     int         device = 0;
     std::string error;
     bool        half_io = false; // half-precision arrays: the plan computes in single precision on scratch copies
+    std::mutex                stage_lock;
+    std::map<void*, StageSet> stage; // by stream
+    ~rocfft_plan_t()
+    {
+        if(!stage.empty())
+            fftrt_device_sync(); // executions in flight may still use the buffers
+        for(auto& kv : stage)
+            kv.second.release();
+    }
 };
 
 struct rocfft_execution_info_t
@@ -469,11 +508,16 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         void*  stream = info ? info->stream : nullptr;
         // the work area of the pass list these buffers get (staged copies are aligned allocations)
         const bool staged_run = plan->half_io || (info && (info->load_cb || info->store_cb));
-        size_t     need       = staged_run ? ep.own_work_bytes()
+        size_t     need       = staged_run ? ep.work_bytes()
                                            : select_exec_plan(ep, in, out, info ? info->workBuffer : nullptr)
                                            .own_work_bytes();
-        void*  work   = nullptr;
-        bool   own    = false;
+        const bool have_cb = info && (info->load_cb || info->store_cb);
+        const bool half_io = plan->half_io;
+        const bool staging = have_cb || half_io;
+        if(staging && static_work)
+            return rocfft_status_failure; // staged copies live in buffers the plan allocates
+        void* work = nullptr;
+        bool  own  = false;
         if(need && static_work)
         {
             size_t have = 0;
@@ -496,7 +540,7 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
                     return rocfft_status_invalid_work_buffer;
                 work = info->workBuffer;
             }
-            else
+            else if(!staging)
             {
                 // no caller-owned scratch: allocate for this call (reference
                 // transform.cpp:424-434); impossible while the stream is being captured
@@ -509,33 +553,23 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         }
         if(pass_ms && fftrt_stream_capturing(stream))
             return rocfft_status_failure;
+        auto cleanup = [&]() {
+            if(own)
+            {
+                fftrt_stream_sync(stream);
+                fftrt_free(work);
+            }
+        };
 
         // Staging.  Load/store callbacks: the input is copied into a scratch buffer of the same
         // layout through the load callback, the plan runs on scratch buffers, and the result
         // goes to the user's buffer through the store callback (two extra element-wise
         // passes; the transform kernels themselves make no indirect calls).  Half precision:
         // the plan computes in single precision on scratch arrays of the same layout, filled
-        // from and written back to the user's half-precision arrays the same way.
-        void*      st_in[2]  = {nullptr, nullptr};
-        void*      st_out[2] = {nullptr, nullptr};
-        const bool have_cb   = info && (info->load_cb || info->store_cb);
-        const bool half_io   = plan->half_io;
-        const bool staging   = have_cb || half_io;
-        if(staging && static_work)
-            return rocfft_status_failure; // staged copies are allocated per call
-        auto       cleanup   = [&]() {
-            if(own || staging)
-                fftrt_stream_sync(stream);
-            if(own)
-                fftrt_free(work);
-            for(int i = 0; i < 2; ++i)
-            {
-                if(st_in[i])
-                    fftrt_free(st_in[i]);
-                if(st_out[i] && st_out[i] != st_in[i])
-                    fftrt_free(st_out[i]);
-            }
-        };
+        // from and written back to the user's half-precision arrays the same way.  The scratch
+        // arrays belong to the plan (one set per stream, see StageSet).
+        void*          st_in[2]  = {nullptr, nullptr};
+        void*          st_out[2] = {nullptr, nullptr};
         fftk_cb_params cin, cout;
         memset(&cin, 0, sizeof(cin));
         memset(&cout, 0, sizeof(cout));
@@ -547,11 +581,8 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         bool       stage_in = false, stage_out = false;
         if(staging)
         {
-            if((have_cb && (in_planar || out_planar || half_io)) || fftrt_stream_capturing(stream))
-            {
-                cleanup();
+            if(have_cb && (in_planar || out_planar || half_io))
                 return rocfft_status_failure;
-            }
             const size_t scalar = ep.precision ? 8 : 4; // of the scratch arrays
             auto         fill   = [&](fftk_cb_params& c, bool input) {
                 size_t off0   = input ? std::max(pr.ioffset[0], pr.ioffset[1]) : std::max(pr.ooffset[0], pr.ooffset[1]);
@@ -571,20 +602,62 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
                 extent += (pr.batch - 1) * (size_t)c.dist;
                 return extent * scalar * ((input ? in_complex : out_complex) ? 2 : 1);
             };
-            const size_t in_bytes  = fill(cin, true);
+            size_t       in_bytes  = fill(cin, true);
             const size_t out_bytes = fill(cout, false);
             stage_in               = ep.inplace || half_io || info->load_cb;
             stage_out              = ep.inplace || half_io || info->store_cb;
-            bool ok                = true;
-            for(int i = 0; i < nin && ok && stage_in; ++i)
-                ok = fftrt_malloc(&st_in[i], ep.inplace ? std::max(in_bytes, out_bytes) : in_bytes) == 0;
-            for(int i = 0; i < nout && ok && stage_out; ++i)
+            if(ep.inplace)
+                in_bytes = std::max(in_bytes, out_bytes);
+            const size_t want_work = (need && !work) ? need : 0;
             {
-                if(ep.inplace)
-                    st_out[i] = st_in[i];
-                else
-                    ok = fftrt_malloc(&st_out[i], out_bytes) == 0;
+                std::lock_guard<std::mutex> guard(plan->stage_lock);
+                StageSet&                   set = plan->stage[stream];
+                const bool fits = (!stage_in || (set.in[0] && set.in_bytes >= in_bytes && (nin < 2 || set.in[1])))
+                                  && (!stage_out || ep.inplace
+                                      || (set.out[0] && set.out_bytes >= out_bytes && (nout < 2 || set.out[1])))
+                                  && (!ep.inplace || set.shared || !set.in[0])
+                                  && set.work_bytes >= want_work;
+                if(!fits)
+                {
+                    // (re)allocate: not while the stream is being captured, and only after
+                    // earlier executions on this stream have let go of the old buffers
+                    if(fftrt_stream_capturing(stream))
+                        return rocfft_status_failure;
+                    fftrt_stream_sync(stream);
+                    set.release();
+                    bool ok = true;
+                    for(int i = 0; i < nin && ok && stage_in; ++i)
+                        ok = fftrt_malloc(&set.in[i], in_bytes) == 0;
+                    set.in_bytes = stage_in ? in_bytes : 0;
+                    set.shared   = ep.inplace;
+                    for(int i = 0; i < nout && ok && stage_out; ++i)
+                    {
+                        if(ep.inplace)
+                            set.out[i] = set.in[i];
+                        else
+                            ok = fftrt_malloc(&set.out[i], out_bytes) == 0;
+                    }
+                    set.out_bytes = stage_out ? (ep.inplace ? in_bytes : out_bytes) : 0;
+                    if(ok && want_work)
+                    {
+                        ok             = fftrt_malloc(&set.work, want_work) == 0;
+                        set.work_bytes = ok ? want_work : 0;
+                    }
+                    if(!ok)
+                    {
+                        set.release();
+                        return rocfft_status_failure;
+                    }
+                }
+                for(int i = 0; i < 2; ++i)
+                {
+                    st_in[i]  = stage_in ? set.in[i] : nullptr;
+                    st_out[i] = stage_out ? set.out[i] : nullptr;
+                }
+                if(want_work)
+                    work = set.work;
             }
+            bool ok = true;
             for(int i = 0; i < nin && ok && stage_in; ++i)
             {
                 cin.store   = 0;
@@ -598,10 +671,7 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
                      == 0;
             }
             if(!ok)
-            {
-                cleanup();
                 return rocfft_status_failure;
-            }
         }
         void* run_in[2]  = {stage_in ? st_in[0] : in[0], stage_in ? st_in[1] : in[1]};
         void* run_out[2] = {stage_out ? st_out[0] : out[0], stage_out ? st_out[1] : out[1]};

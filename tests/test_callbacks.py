@@ -101,3 +101,78 @@ def test_callbacks_on_the_gpu(gpu_lib, which):
     for kind, lengths, batch, precision, kw in CASES:
         print("callback case", kind, lengths, precision, kw, which, flush=True)
         check_case(gpu_lib, H.TorchBackend(), cblib, kind, lengths, batch, precision, kw, which)
+
+
+@pytest.mark.gpu
+def test_staged_executions_replay_from_a_graph(gpu_lib):
+    """Executions that stage through copies (callbacks, half precision) keep their copies in
+    buffers the plan owns per stream: the first execution on a stream allocates them, later
+    ones allocate nothing and can be captured.  Every replay is checked against an eager
+    execution, with eager work between the replays."""
+    import torch
+
+    lib = gpu_lib
+    dev = torch.device("cuda:0")
+    cblib = callback_library("libcb_device.so")
+    n, batch = 4096, 6
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.view_as_complex(torch.rand((batch, n, 2), generator=gen, device=dev) - 0.5)
+    scales = torch.tensor([S_LOAD, S_STORE], dtype=torch.float32, device=dev)
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], batch, lib=lib)
+    side = torch.cuda.Stream()
+
+    def new_info():
+        info = B.ExecutionInfo(lib).set_stream(side.cuda_stream)
+        info.set_load_callback(cblib.cb_get(0, 1, 0), scales[0:].data_ptr())
+        info.set_store_callback(cblib.cb_get(1, 1, 0), scales[1:].data_ptr())
+        return info
+
+    xin = x.clone()
+    y = torch.zeros_like(x)
+    info = new_info()
+    torch.cuda.synchronize()
+    # before the plan has buffers for this stream, a captured execution is refused
+    g0 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g0, stream=side):
+            refused = plan.execute_status([xin.data_ptr()], [y.data_ptr()], info)
+    assert refused == B.STATUS_FAILURE
+    # the first eager execution on the stream allocates them
+    plan.execute([xin.data_ptr()], [y.data_ptr()], info)
+    side.synchronize()
+    ref = torch.fft.fft(x, dim=1) * (S_LOAD * S_STORE)
+    assert (torch.linalg.vector_norm(y - ref) / torch.linalg.vector_norm(ref)).item() < 1e-5
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            plan.execute([xin.data_ptr()], [y.data_ptr()], info)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        xin.copy_(x * (rep + 2))
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        err = (torch.linalg.vector_norm(y - ref * (rep + 2)) / torch.linalg.vector_norm(ref)).item()
+        assert err < 1e-5 * (rep + 2), (rep, err)
+
+    # half precision the same way
+    hplan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256], 4, lib=lib)
+    xh = (torch.rand((4, 256, 2), generator=gen, device=dev) - 0.5).to(torch.float16)
+    yh = torch.zeros_like(xh)
+    hinfo = B.ExecutionInfo(lib).set_stream(side.cuda_stream)
+    hplan.execute([xh.data_ptr()], [yh.data_ptr()], hinfo)
+    side.synchronize()
+    want = yh.clone()
+    gh = torch.cuda.CUDAGraph()
+    yh.zero_()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(gh, stream=side):
+            hplan.execute([xh.data_ptr()], [yh.data_ptr()], hinfo)
+    torch.cuda.synchronize()
+    for rep in range(2):
+        yh.zero_()
+        torch.cuda.synchronize()
+        gh.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(yh, want), rep
