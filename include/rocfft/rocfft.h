@@ -60,8 +60,9 @@ typedef enum rocfft_transform_type_e
     rocfft_transform_type_real_inverse    = 3
 } rocfft_transform_type;
 
-/* Precision (reference rocfft.h:100-105). Half precision is not implemented:
-   plan creation returns rocfft_status_failure for it. */
+/* Precision (reference rocfft.h:100-105). Half precision keeps the layouts of
+   the plan description; its arrays hold IEEE half values, the arithmetic runs in
+   single precision on copies the plan owns and the result is rounded back. */
 typedef enum rocfft_precision_e
 {
     rocfft_precision_single = 0,

@@ -106,78 +106,57 @@ struct rocfft_brick_t
 // ---------------------------------------------------------------------------
 // defaults and validation
 
-// fills unset array types, strides and distances (reference plan.cpp:87-197)
-static void init_defaults(rocfft_plan_description_t& d, rocfft_transform_type type,
-                          rocfft_result_placement placement, const std::vector<size_t>& lengths,
-                          const std::vector<size_t>& outputLengths)
+// What a plan description may leave unset on one side (input or output) of a transform, and
+// the rule of the API that completes it (the contract of the reference's defaults,
+// library/src/plan.cpp:87-197; see also the in-place real layouts of rocfft.h:107-112):
+//   array type  a real transform has one real and one Hermitian side, a complex one two
+//               interleaved complex sides;
+//   strides     packed: dimension d steps over the rows of the dimensions below it.  The real side
+//               of an in-place real transform lies over the Hermitian rows, so its row 0 takes the
+//               2 (n0/2 + 1) reals that row covers instead of n0;
+//   distance    the extent of one transform, i.e. last length x last stride -- for rank 1 laid over
+//               the Hermitian row as above.
+enum SideRole
 {
-    const size_t rank = lengths.size();
-    if(d.inArrayType == rocfft_array_type_unset)
+    SIDE_COMPLEX,
+    SIDE_REAL,
+    SIDE_HERMITIAN
+};
+
+static void complete_side(rocfft_array_type& type, std::vector<size_t>& stride, size_t& dist, SideRole role,
+                          bool laid_over_hermitian, const std::vector<size_t>& array_len, size_t hermitian_row)
+{
+    if(type == rocfft_array_type_unset)
+        type = role == SIDE_REAL        ? rocfft_array_type_real
+               : role == SIDE_HERMITIAN ? rocfft_array_type_hermitian_interleaved
+                                        : rocfft_array_type_complex_interleaved;
+    const size_t rank = array_len.size();
+    const size_t row0 = laid_over_hermitian ? 2 * hermitian_row : array_len[0];
+    if(stride.empty())
     {
-        if(type == rocfft_transform_type_real_forward)
-            d.inArrayType = rocfft_array_type_real;
-        else if(type == rocfft_transform_type_real_inverse)
-            d.inArrayType = rocfft_array_type_hermitian_interleaved;
-        else
-            d.inArrayType = rocfft_array_type_complex_interleaved;
-    }
-    if(d.outArrayType == rocfft_array_type_unset)
-    {
-        if(type == rocfft_transform_type_real_forward)
-            d.outArrayType = rocfft_array_type_hermitian_interleaved;
-        else if(type == rocfft_transform_type_real_inverse)
-            d.outArrayType = rocfft_array_type_real;
-        else
-            d.outArrayType = rocfft_array_type_complex_interleaved;
-    }
-    const bool inplace = placement == rocfft_placement_inplace;
-    if(d.inStrides.empty())
-    {
-        d.inStrides.push_back(1);
-        if(type == rocfft_transform_type_real_forward && inplace)
+        size_t step = 1;
+        for(size_t d = 0; d < rank; ++d)
         {
-            // rows padded so that the Hermitian output fits over the real input
-            size_t dist = 2 * outputLengths[0];
-            for(size_t i = 1; i < rank; ++i)
-            {
-                d.inStrides.push_back(dist);
-                dist *= lengths[i];
-            }
+            stride.push_back(step);
+            step *= d == 0 ? row0 : array_len[d];
         }
-        else
-            for(size_t i = 1; i < rank; ++i)
-                d.inStrides.push_back(lengths[i - 1] * d.inStrides[i - 1]);
     }
-    if(d.outStrides.empty())
-    {
-        d.outStrides.push_back(1);
-        if(type == rocfft_transform_type_real_inverse && inplace)
-        {
-            size_t dist = 2 * lengths[0];
-            for(size_t i = 1; i < rank; ++i)
-            {
-                d.outStrides.push_back(dist);
-                dist *= lengths[i];
-            }
-        }
-        else
-            for(size_t i = 1; i < rank; ++i)
-                d.outStrides.push_back(outputLengths[i - 1] * d.outStrides[i - 1]);
-    }
-    if(d.inDist == 0)
-    {
-        if(type == rocfft_transform_type_real_forward && rank == 1 && inplace)
-            d.inDist = 2 * (lengths[0] / 2 + 1) * d.inStrides[0];
-        else
-            d.inDist = lengths[rank - 1] * d.inStrides[rank - 1];
-    }
-    if(d.outDist == 0)
-    {
-        if(type == rocfft_transform_type_real_inverse && rank == 1 && inplace)
-            d.outDist = 2 * lengths[0] * d.outStrides[0];
-        else
-            d.outDist = outputLengths[rank - 1] * d.outStrides[rank - 1];
-    }
+    if(dist == 0)
+        dist = (rank == 1 && laid_over_hermitian) ? row0 * stride[0] : array_len[rank - 1] * stride[rank - 1];
+}
+
+static void init_defaults(rocfft_plan_description_t& d, rocfft_transform_type type,
+                          rocfft_result_placement placement, const std::vector<size_t>& in_len,
+                          const std::vector<size_t>& out_len)
+{
+    const bool   inplace = placement == rocfft_placement_inplace;
+    const bool   fwd     = type == rocfft_transform_type_real_forward;
+    const bool   inv     = type == rocfft_transform_type_real_inverse;
+    const size_t herm    = fwd ? out_len[0] : in_len[0]; // bins per Hermitian row (real transforms)
+    complete_side(d.inArrayType, d.inStrides, d.inDist, fwd ? SIDE_REAL : inv ? SIDE_HERMITIAN : SIDE_COMPLEX,
+                  fwd && inplace, in_len, herm);
+    complete_side(d.outArrayType, d.outStrides, d.outDist, fwd ? SIDE_HERMITIAN : inv ? SIDE_REAL : SIDE_COMPLEX,
+                  inv && inplace, out_len, herm);
 }
 
 // transform type, array types and placement must agree (reference plan.cpp:729-779)

@@ -521,8 +521,9 @@ struct BigDirectChunks
 //   request the copy global -> LDS of the prefetched part of i + 1; pass 2;
 //   wait for that copy; stores of i.
 // Measured on MI355X and not kept: requesting the direct part of i + 1 between the stores of i
-// (slower: loads queue behind the stores), nontemporal loads and stores (no gain; slower for
-// the 8-byte aligned rows of 32769 bins, whose partial lines no longer merge in L2).
+// (slower: loads queue behind the stores) or ahead of them (no change), nontemporal loads and
+// stores (no gain; slower for the 8-byte aligned rows of 32769 bins, whose partial lines no
+// longer merge in L2).
 template <int MODE, bool INV>
 __global__ __launch_bounds__(BIG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void big32k_stream_kernel(
     const big_params p, const uint32_t total)
