@@ -15,6 +15,7 @@
 #include "butterfly.h"
 #include "gpu_rt.h"
 #include "kparams.h"
+#include "lds_limit.h"
 #include <hip/hip_runtime.h>
 #include <algorithm>
 #include <atomic>
@@ -802,32 +803,12 @@ __global__ __launch_bounds__(BIG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 
 constexpr size_t BIG_LDS_BYTES = (size_t)(BIG_L + BIG_L / 32 + 32) * sizeof(float);
 constexpr int    BIG_MAX_DEVICES = 64;
 
-// Raises a kernel's dynamic-LDS limit once per device.  The result is kept per device: a
-// failed attempt is tried again by the next launch and reported to every caller until it succeeds.
-template <typename K>
-int big_allow_lds(K kernel, std::atomic<int>* done, int dev)
-{
-    if(dev < 0 || dev >= BIG_MAX_DEVICES)
-        return (int)hipErrorInvalidDevice;
-    if(done[dev].load(std::memory_order_acquire))
-        return 0;
-    int rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if(rc == 0)
-        done[dev].store(1, std::memory_order_release);
-    return rc;
-}
-
 template <int MODE>
 int launch_big(const big_params& p, uint32_t grid, hipStream_t stream)
 {
-    auto                    kernel = big32k_kernel<MODE>;
-    static std::atomic<int> done[BIG_MAX_DEVICES];
-    int                     dev = 0;
-    int                     rc  = (int)hipGetDevice(&dev);
-    if(rc == 0)
-        rc = big_allow_lds(kernel, done, dev);
-    if(rc)
+    auto               kernel = big32k_kernel<MODE>;
+    static FftLdsLimit limit;
+    if(int rc = limit.allow(kernel))
         return rc;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(BIG_THREADS), BIG_LDS_BYTES, stream, p);
     return (int)hipGetLastError();
@@ -852,13 +833,12 @@ int big_compute_units(int dev)
 template <int MODE, bool INV>
 int launch_big_stream(const big_params& p, uint32_t total, hipStream_t stream)
 {
-    auto                    kernel = big32k_stream_kernel<MODE, INV>;
-    static std::atomic<int> done[BIG_MAX_DEVICES];
-    int                     dev = 0;
-    int                     rc  = (int)hipGetDevice(&dev);
-    if(rc == 0)
-        rc = big_allow_lds(kernel, done, dev);
-    if(rc)
+    auto               kernel = big32k_stream_kernel<MODE, INV>;
+    static FftLdsLimit limit;
+    if(int rc = limit.allow(kernel))
+        return rc;
+    int dev = 0;
+    if(int rc = (int)hipGetDevice(&dev))
         return rc;
     const int units = big_compute_units(dev);
     if(units <= 0)

@@ -5,6 +5,7 @@
 // translation unit instantiates the kernels of its slice of the list, and slice 0 also
 // holds the lookup over all slices.
 #include "fast_core.h"
+#include "lds_limit.h"
 #include "fast_registry.h"
 #include "gpu_rt.h"
 #include <hip/hip_runtime.h>
@@ -45,15 +46,8 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* str
     auto kernel = fast_tile_kernel<T, Cfg, MODE>;
     if(lds_bytes > 64 * 1024)
     {
-        static std::once_flag once[16];
-        int                   dev = 0;
-        (void)hipGetDevice(&dev);
-        int rc = 0;
-        std::call_once(once[dev & 15], [&]() {
-            rc = (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        });
-        if(rc)
+        static FftLdsLimit limit;
+        if(int rc = limit.allow(kernel))
             return rc;
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(p->nthreads), lds_bytes, (hipStream_t)stream, *p);

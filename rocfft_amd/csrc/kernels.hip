@@ -1,5 +1,6 @@
 // kernels.hip -- gfx950 kernels and the HIP side of the C-ABI runtime layer.
 #include "gpu_rt.h"
+#include "lds_limit.h"
 #include "tile_core.h"
 #include <hip/hip_runtime.h>
 #include <mutex>
@@ -108,28 +109,14 @@ __global__ __launch_bounds__(256) void real_pre_kernel(const fftk_real_params p)
 
 constexpr size_t MAX_LDS_BYTES = 160 * 1024;
 
-template <typename K>
-int raise_lds_limit(K kernel)
-{
-    return (int)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)MAX_LDS_BYTES);
-}
-
 template <typename T, bool VEC, int BLK>
 int launch_tile_t(const fftk_params* p, uint32_t grid, size_t lds_bytes, hipStream_t stream)
 {
     auto kernel = tile_fft_kernel<T, VEC, BLK>;
     if(lds_bytes > 64 * 1024)
     {
-        // raised once per kernel and device; hipFuncSetAttribute is not a
-        // stream operation, so it is legal during graph capture
-        static std::once_flag once[16];
-        int                   dev = 0;
-        (void)hipGetDevice(&dev);
-        int rc = 0;
-        std::call_once(once[dev & 15], [&]() { rc = raise_lds_limit(kernel); });
-        if(rc)
+        static FftLdsLimit limit;
+        if(int rc = limit.allow(kernel, (int)MAX_LDS_BYTES))
             return rc;
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(p->nthreads), lds_bytes, stream, *p);

@@ -769,6 +769,16 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         else if(w_lds < w_run && per_tile <= LDS_WIDE_BYTES)
             w_lds = std::max(w_lds, std::min(w_run, floor_pow2(LDS_WIDE_BYTES / per_tile)));
         W = std::min(std::min<uint32_t>(64, w_threads), std::min(w_lds, w_cap));
+        // experiment switch: ROCFFT_AMD_COLW=<w> asks for column tiles w transforms wide (when
+        // threads and LDS allow)
+        static const char* colw = getenv("ROCFFT_AMD_COLW");
+        if(colw)
+        {
+            const uint32_t want = (uint32_t)atoi(colw);
+            const uint32_t fit  = std::min(w_threads, floor_pow2((uint32_t)(LDS_WIDE_BYTES / per_tile)));
+            if(want >= 1)
+                W = std::min(std::min(want, fit), w_cap);
+        }
     }
     else
     {

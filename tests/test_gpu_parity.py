@@ -261,6 +261,47 @@ def test_c2r_ignores_imaginary_dc_and_nyquist(gpu):
         assert np.array_equal(y1, y2), n
 
 
+def test_streaming_one_workgroup_kernel_batches_and_layouts(gpu):
+    """The one-workgroup 32768-point kernel walks through the transforms of a launch, a workgroup
+    taking every G-th one and prefetching its next: batch counts below, at and above the
+    number of workgroups (1024 on MI355X), rows that alternate between 16- and 8-byte alignment
+    (32769 bins), padded distances, a second dimension, scaling, both complex directions."""
+    lib, be = gpu
+    torch = be.torch
+    # against the checker: few transforms, every mode, odd row alignments
+    for kind, lengths, batch, kw in [
+            (B.REAL_FORWARD, [65536], 1, {}), (B.REAL_INVERSE, [65536], 1, {}),
+            (B.REAL_FORWARD, [65536], 5, {"scale": 0.5}), (B.REAL_INVERSE, [65536], 5, {"scale": 1.0 / 65536}),
+            (B.COMPLEX_FORWARD, [32768], 3, {}), (B.COMPLEX_INVERSE, [32768], 3, {"scale": 2.0}),
+            (B.COMPLEX_FORWARD, [32768], 2, {"inplace": True}),
+            (B.REAL_FORWARD, [65536], 3, {"in_strides": [1], "in_dist": 65536 + 12, "out_strides": [1], "out_dist": 32769 + 3}),
+            (B.REAL_INVERSE, [65536], 3, {"in_strides": [1], "in_dist": 32769 + 2, "out_strides": [1], "out_dist": 65536 + 4}),
+            (B.REAL_FORWARD, [65536, 3], 2, {}), (B.REAL_INVERSE, [65536, 3], 2, {}), (B.COMPLEX_FORWARD, [32768, 2], 2, {})]:
+        H.check(lib, be, kind, lengths, batch, B.SINGLE, **kw)
+    # many transforms: round trip and a cross-check of a few rows against torch.fft
+    n = 65536
+    for batch in (255, 1023, 1024, 1025, 2500):
+        x = (inputs.torch_uniform01(torch, be.dev, 40 + batch, 0, n * batch) * 2 - 1).to(torch.float32).reshape(batch, n)
+        h = torch.full((batch, n // 2 + 1), float("nan"), dtype=torch.complex64, device=be.dev)
+        y = torch.full((batch, n), float("nan"), dtype=torch.float32, device=be.dev)
+        fwd = B.Plan(B.NOTINPLACE, B.REAL_FORWARD, B.SINGLE, [n], batch, lib=lib)
+        inv = B.Plan(B.NOTINPLACE, B.REAL_INVERSE, B.SINGLE, [n], batch, lib=lib)
+        fwd.execute([x.data_ptr()], [h.data_ptr()])
+        inv.execute([h.data_ptr()], [y.data_ptr()])
+        torch.cuda.synchronize()
+        rows = sorted(set([0, 1, batch // 2, batch - 2, batch - 1]))
+        ref = torch.fft.rfft(x[rows].double(), dim=1)
+        l2, li = tnorm(torch, h[rows], ref)
+        assert l2 <= 1e-5 and li <= 1e-5, (batch, l2, li)
+        l2, li = tnorm(torch, y / n, x)
+        assert l2 <= 1e-5 and li <= 1e-5, (batch, l2, li)
+        # every row, cheaply: Parseval per row
+        e_in = (x.double() ** 2).sum(dim=1)
+        hh = torch.view_as_real(h).double()
+        e_out = (2 * (hh ** 2).sum(dim=(1, 2)) - hh[:, 0, 0] ** 2 - hh[:, -1, 0] ** 2) / n
+        assert ((e_out / e_in - 1).abs().max().item()) < 1e-5, batch
+
+
 def test_buffers_aligned_to_a_scalar_only(gpu):
     """Base pointers offset by one scalar.  The kernels that move (re, im) pairs with one
     access have no form for such buffers; plans that use them carry a second pass list made
