@@ -485,14 +485,28 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         if((planar(pr.in_type) && !in[1]) || (planar(pr.out_type) && !out[1]))
             return rocfft_status_failure;
         void*  stream = info ? info->stream : nullptr;
+        // Load/store callbacks run inside the first and last kernel when those have a callback
+        // form (interleaved or real arrays); otherwise, and for half precision, the arrays are
+        // staged through copies.
+        const bool    have_cb = info && (info->load_cb || info->store_cb);
+        const bool    half_io = plan->half_io;
+        ExecCallbacks ecb;
+        bool          fused = false;
+        if(have_cb && !half_io && !planar(pr.in_type) && !planar(pr.out_type))
+        {
+            ecb.load_fn     = info->load_cb;
+            ecb.load_data   = info->load_cb_data;
+            ecb.store_fn    = info->store_cb;
+            ecb.store_data  = info->store_cb_data;
+            ecb.in_complex  = pr.in_type != rocfft_array_type_real;
+            ecb.out_complex = pr.out_type != rocfft_array_type_real;
+            fused           = callbacks_fusable(ep, in, out, info->workBuffer, ecb);
+        }
+        const bool staging = half_io || (have_cb && !fused);
         // the work area of the pass list these buffers get (staged copies are aligned allocations)
-        const bool staged_run = plan->half_io || (info && (info->load_cb || info->store_cb));
-        size_t     need       = staged_run ? ep.work_bytes()
-                                           : select_exec_plan(ep, in, out, info ? info->workBuffer : nullptr)
-                                           .own_work_bytes();
-        const bool have_cb = info && (info->load_cb || info->store_cb);
-        const bool half_io = plan->half_io;
-        const bool staging = have_cb || half_io;
+        size_t need = staging ? ep.work_bytes()
+                              : select_exec_plan(ep, in, out, info ? info->workBuffer : nullptr, fused ? &ecb : nullptr)
+                                    .own_work_bytes();
         if(staging && static_work)
             return rocfft_status_failure; // staged copies live in buffers the plan allocates
         void* work = nullptr;
@@ -654,7 +668,7 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         }
         void* run_in[2]  = {stage_in ? st_in[0] : in[0], stage_in ? st_in[1] : in[1]};
         void* run_out[2] = {stage_out ? st_out[0] : out[0], stage_out ? st_out[1] : out[1]};
-        rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms);
+        rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms, fused ? &ecb : nullptr);
         for(int i = 0; i < nout && st == rocfft_status_success && stage_out; ++i)
         {
             cout.store   = 1;

@@ -41,6 +41,28 @@ enum fftk_flags
     FFTK_F_CHIRP_CONJ    = 1 << 5  // use the conjugate chirp (inverse-direction Bluestein)
 };
 
+// User load/store callbacks of an execution (reference library/include/rocfft/rocfft.h:533-612),
+// called from inside the first and the last kernel of a plan:
+//   T    load_cb (T* data, size_t offset, void* cbdata, void* sharedMem);
+//   void store_cb(T* data, size_t offset, T element, void* cbdata, void* sharedMem);
+// data is the buffer pointer given to rocfft_execute, offset counts elements of the array's type
+// (real scalars, or complex pairs for interleaved complex arrays).  The kernels address scalars
+// relative to their own base pointers; *_off is the distance of that base from the user's
+// pointer, in scalars.  A null function pointer means plain memory access.
+struct fftk_cb
+{
+    const void* load_fn;
+    void*       load_data;
+    const void* in_base;    // the user's input pointer
+    int64_t     in_off;     // scalars from in_base to the kernel's input base
+    uint32_t    in_complex; // 1: the callback's element is a complex pair
+    uint32_t    out_complex;
+    const void* store_fn;
+    void*       store_data;
+    void*       out_base;
+    int64_t     out_off;
+};
+
 struct fftk_params
 {
     // transform
@@ -100,6 +122,7 @@ struct fftk_params
     const void* convb;              // spectrum the tile is multiplied with in CONV mode
     uint32_t    convb_qs;           // its index = j + q*convb_qs
     double      scale;
+    struct fftk_cb cb; // run-time-schedule kernel only
 };
 
 // standalone even-length real post-/pre-processing over natural-order rows
@@ -120,6 +143,7 @@ struct fftk_real_params
     const void* half_tw; // e^{-2 pi i j/(2L)}, j in [0, L/2]
     double      scale;
     uint32_t    use_scale;
+    struct fftk_cb cb; // post: store side (Hermitian bins); pre: load side
 };
 
 // element-wise row copy between array kinds: real -> complex, complex -> real, Hermitian half
@@ -143,6 +167,7 @@ struct fftk_copy_params
     void*       d1;
     double      scale;
     uint32_t    use_scale;
+    struct fftk_cb cb;
 };
 
 // Copy of every element of a transform's input (or output) between the user's buffer and a

@@ -2619,10 +2619,35 @@ static bool aligned(const void* p, size_t a)
     return ((uintptr_t)p % a) == 0;
 }
 
-const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work)
+// a pass the run-time-schedule kernels can run with a callback on its load (first) or store (last) side
+static bool pass_takes_callback(const PassRec& r, bool load_side)
+{
+    switch(r.kind)
+    {
+    case PASS_TILE:
+        return r.kp.nthreads <= 512 && !r.src.planar && !r.dst.planar;
+    case PASS_REAL_POST:
+        return !load_side;
+    case PASS_REAL_PRE:
+        return load_side;
+    case PASS_COPY:
+        return true;
+    default:
+        return false;
+    }
+}
+
+const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work,
+                                 const ExecCallbacks* cb)
 {
     if(!plan.unaligned)
         return plan;
+    // callbacks run inside the first and last kernel: when the plan's own is a kernel without
+    // callback form, the other list (run-time-schedule kernels only) takes over
+    if(cb && !plan.passes.empty()
+       && ((cb->load_fn && !pass_takes_callback(plan.passes.front(), true))
+           || (cb->store_fn && !pass_takes_callback(plan.passes.back(), false))))
+        return *plan.unaligned;
     const size_t scalar = plan.precision ? 8 : 4;
     auto         base   = [&](const IoRef& io) -> const char* {
         switch(io.buf)
@@ -2650,20 +2675,61 @@ const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* 
     return plan;
 }
 
+bool callbacks_fusable(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work,
+                       const ExecCallbacks& cb)
+{
+    const ExecPlan& chosen = select_exec_plan(plan, in, out, work, &cb);
+    if(chosen.passes.empty())
+        return false;
+    if(cb.load_fn && !pass_takes_callback(chosen.passes.front(), true))
+        return false;
+    if(cb.store_fn && !pass_takes_callback(chosen.passes.back(), false))
+        return false;
+    return true;
+}
+
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
-                            void* stream, float* pass_ms)
+                            void* stream, float* pass_ms, const ExecCallbacks* cb)
 {
     {
-        const ExecPlan& chosen = select_exec_plan(plan, in, out, work);
+        const ExecPlan& chosen = select_exec_plan(plan, in, out, work, cb);
         if(&chosen != &plan)
         {
             // (per-pass timings describe the primary pass list: not reported for the other one)
             if(pass_ms)
                 for(size_t i = 0; i < plan.passes.size(); ++i)
                     pass_ms[i] = -1.0f;
-            return run_exec_plan(chosen, in, out, work, stream, nullptr);
+            return run_exec_plan(chosen, in, out, work, stream, nullptr, cb);
         }
     }
+    // the callback descriptor of a pass: the load callback belongs to the first pass, the
+    // store callback to the last one; every other access is plain
+    const size_t npass = plan.passes.size();
+    auto         cb_of = [&](size_t index, const IoRef& src, const IoRef& dst, fftk_cb& d) {
+        memset(&d, 0, sizeof(d));
+        if(!cb)
+            return false;
+        bool any = false;
+        if(cb->load_fn && index == 0)
+        {
+            d.load_fn    = cb->load_fn;
+            d.load_data  = cb->load_data;
+            d.in_base    = in[0];
+            d.in_off     = src.off0;
+            d.in_complex = cb->in_complex ? 1 : 0;
+            any          = true;
+        }
+        if(cb->store_fn && index + 1 == npass)
+        {
+            d.store_fn    = cb->store_fn;
+            d.store_data  = cb->store_data;
+            d.out_base    = out[0];
+            d.out_off     = dst.off0;
+            d.out_complex = cb->out_complex ? 1 : 0;
+            any           = true;
+        }
+        return any;
+    };
     const size_t scalar = plan.precision ? 8 : 4;
     char*        tmp    = static_cast<char*>(work);
     char*        blu    = tmp ? tmp + plan.tmp_elems * plan.elem_bytes : nullptr;
@@ -2732,6 +2798,12 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
         if(!resolve(rec.src, s0, s1) || !resolve(rec.dst, d0, d1))
             return rocfft_status_failure;
         int rc;
+        if(rec.kind == PASS_BIG || rec.kind == PASS_2D)
+        {
+            fftk_cb none;
+            if(cb_of(pass_index, rec.src, rec.dst, none))
+                return rocfft_status_failure; // these kernels have no callback form
+        }
         if(rec.kind == PASS_BIG)
         {
             fftk_big_params q = rec.bp;
@@ -2763,6 +2835,7 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             c.s1               = s1;
             c.d0               = d0;
             c.d1               = d1;
+            cb_of(pass_index, rec.src, rec.dst, c.cb);
             rc                 = fftrt_launch_copy(&c, plan.precision, stream);
         }
         else if(rec.kind == PASS_TILE)
@@ -2774,7 +2847,16 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             k.out1        = d1;
             bool vec = rec.vec_ok && aligned(s0, plan.elem_bytes) && aligned(d0, plan.elem_bytes);
             k.lean   = (rec.lean_ok && vec) ? 1 : 0;
-            if(rec.lean_real)
+            const bool with_cb = cb_of(pass_index, rec.src, rec.dst, k.cb);
+            if(with_cb)
+            {
+                // the run-time-schedule kernel runs the same schedule and calls the callbacks
+                if(!pass_takes_callback(rec, pass_index == 0 && cb->load_fn))
+                    return rocfft_status_failure;
+                k.fast = 0;
+                k.lean = 0;
+            }
+            if(rec.lean_real && !with_cb)
             {
                 // the real side needs scalar alignment only
                 const bool in_ok  = aligned(s0, k.load_op == FFTK_LOAD_REAL ? plan.elem_bytes / 2 : plan.elem_bytes);
@@ -2786,6 +2868,9 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
         else
         {
             fftk_real_params r = rec.rp;
+            if(cb_of(pass_index, rec.src, rec.dst, r.cb)
+               && !pass_takes_callback(rec, pass_index == 0 && cb->load_fn))
+                return rocfft_status_failure;
             if(rec.kind == PASS_REAL_POST)
             {
                 r.z0  = s0;

@@ -122,17 +122,37 @@ struct ExecPlan
 // null device pointers), so the planner can be exercised without a GPU.
 rocfft_status build_exec_plan(const Problem& prob, ExecPlan& plan, bool dry_run, std::string& err);
 
+// Load/store callbacks of one execution (device function pointers with the reference's
+// signatures, library/include/rocfft/rocfft.h:533-612).  They are called from inside the first
+// and the last kernel of the pass list; those two run as the run-time-schedule kernels, which
+// have the callback form of every load and store.
+struct ExecCallbacks
+{
+    void* load_fn     = nullptr;
+    void* load_data   = nullptr;
+    void* store_fn    = nullptr;
+    void* store_data  = nullptr;
+    bool  in_complex  = false; // the callback's element is a complex pair (interleaved arrays)
+    bool  out_complex = false;
+};
+
 // Enqueues every pass on `stream`.  in/out hold one pointer (interleaved, real)
 // or two (planar).  `work` must hold plan.work_bytes() bytes when that is non-zero.
 // When pass_ms is not null every pass is bracketed by events and its duration in
 // milliseconds is written there (the call then waits for the stream).
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
-                            void* stream, float* pass_ms = nullptr);
+                            void* stream, float* pass_ms = nullptr, const ExecCallbacks* cb = nullptr);
 
 // The pass list run_exec_plan will use for these buffers: the plan itself, or its `unaligned`
 // list when a buffer fails the alignment one of the plan's passes needs.  `work` may be null
 // (not allocated yet: allocations are aligned).
-const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work);
+const ExecPlan& select_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work,
+                                 const ExecCallbacks* cb = nullptr);
+
+// Can the pass list these buffers get call the callbacks from inside its first and last kernel?
+// (If not, the caller stages the arrays through copies instead.)
+bool callbacks_fusable(const ExecPlan& plan, void* const in[2], void* const out[2], const void* work,
+                       const ExecCallbacks& cb);
 
 // drops cached tables that no plan uses any more
 void table_cache_clear();

@@ -76,11 +76,80 @@ FFT_DEV uint32_t lds_addr(const fftk_params& p, uint32_t w, uint32_t j)
     return w * p.pitch + j + (j >> p.padshift);
 }
 
+// ---- user callbacks.  `off` counts scalars from the kernel's base pointer of that side.
+template <typename T>
+FFT_DEV T cb_load_scalar(const fftk_cb& cb, int64_t off)
+{
+    typedef T (*fn_t)(T*, size_t, void*, void*);
+    return reinterpret_cast<fn_t>(const_cast<void*>(cb.load_fn))(
+        static_cast<T*>(const_cast<void*>(cb.in_base)), (size_t)(cb.in_off + off), cb.load_data, nullptr);
+}
+template <typename T>
+FFT_DEV typename cplx_of<T>::type cb_load_pair(const fftk_cb& cb, int64_t off)
+{
+    typedef typename cplx_of<T>::type C;
+    typedef C (*fn_t)(C*, size_t, void*, void*);
+    return reinterpret_cast<fn_t>(const_cast<void*>(cb.load_fn))(
+        static_cast<C*>(const_cast<void*>(cb.in_base)), (size_t)((cb.in_off + off) >> 1), cb.load_data, nullptr);
+}
+template <typename T>
+FFT_DEV void cb_store_scalar(const fftk_cb& cb, int64_t off, T v)
+{
+    typedef void (*fn_t)(T*, size_t, T, void*, void*);
+    reinterpret_cast<fn_t>(const_cast<void*>(cb.store_fn))(static_cast<T*>(cb.out_base), (size_t)(cb.out_off + off), v,
+                                                            cb.store_data, nullptr);
+}
+template <typename T>
+FFT_DEV void cb_store_pair(const fftk_cb& cb, int64_t off, typename cplx_of<T>::type v)
+{
+    typedef typename cplx_of<T>::type C;
+    typedef void (*fn_t)(C*, size_t, C, void*, void*);
+    reinterpret_cast<fn_t>(const_cast<void*>(cb.store_fn))(static_cast<C*>(cb.out_base), (size_t)((cb.out_off + off) >> 1), v,
+                                                            cb.store_data, nullptr);
+}
+// One element whose parts lie at re0[off] and im0[off] (im0 = re0 + a few scalars for
+// interleaved and real-pair layouts), through the load callback when there is one.
+template <typename T>
+FFT_DEV typename cplx_of<T>::type cb_or_load(const fftk_cb& cb, const T* re0, const T* im0, int64_t off)
+{
+    typename cplx_of<T>::type v;
+    if(cb.load_fn)
+    {
+        if(cb.in_complex)
+            return cb_load_pair<T>(cb, off);
+        v.x = cb_load_scalar<T>(cb, off);
+        v.y = cb_load_scalar<T>(cb, off + (im0 - re0));
+        return v;
+    }
+    v.x = re0[off];
+    v.y = im0[off];
+    return v;
+}
+template <typename T>
+FFT_DEV void cb_or_store(const fftk_cb& cb, T* re0, T* im0, int64_t off, typename cplx_of<T>::type v)
+{
+    if(cb.store_fn)
+    {
+        if(cb.out_complex)
+            cb_store_pair<T>(cb, off, v);
+        else
+        {
+            cb_store_scalar<T>(cb, off, v.x);
+            cb_store_scalar<T>(cb, off + (im0 - re0), v.y);
+        }
+        return;
+    }
+    re0[off] = v.x;
+    im0[off] = v.y;
+}
+
 template <typename T, bool VEC>
 FFT_DEV typename cplx_of<T>::type load_elem(const fftk_params& p, int64_t off)
 {
     typedef typename cplx_of<T>::type C;
-    C                                 v;
+    if(p.cb.load_fn)
+        return cb_or_load<T>(p.cb, static_cast<const T*>(p.in0), static_cast<const T*>(p.in1), off);
+    C v;
     if(VEC)
         v = *reinterpret_cast<const C*>(static_cast<const T*>(p.in0) + off);
     else
@@ -95,6 +164,11 @@ template <typename T, bool VEC>
 FFT_DEV void store_elem(const fftk_params& p, int64_t off, typename cplx_of<T>::type v)
 {
     typedef typename cplx_of<T>::type C;
+    if(p.cb.store_fn)
+    {
+        cb_or_store<T>(p.cb, static_cast<T*>(p.out0), static_cast<T*>(p.out1), off, v);
+        return;
+    }
     if(VEC)
         *reinterpret_cast<C*>(static_cast<T*>(p.out0) + off) = v;
     else
@@ -156,7 +230,8 @@ FFT_DEV typename cplx_of<T>::type
     {
         int64_t base = c.ibase + (int64_t)w * p.w_is;
         if(p.load_op == FFTK_LOAD_REAL)
-            v.x = static_cast<const T*>(p.in0)[base + (int64_t)j * p.t_is];
+            v.x = p.cb.load_fn ? cb_load_scalar<T>(p.cb, base + (int64_t)j * p.t_is)
+                               : static_cast<const T*>(p.in0)[base + (int64_t)j * p.t_is];
         else if(p.load_op == FFTK_LOAD_HERM_EXPAND)
         {
             // logical length n_in; bins above n_in/2 are the conjugate mirror,
@@ -387,7 +462,12 @@ FFT_DEV void emit_elem(const fftk_params& p, const TileCtx<T>& c, uint32_t w, ui
     }
     int64_t off = c.obase + (int64_t)j * p.t_os + (int64_t)w * p.w_os;
     if(p.store_op == FFTK_STORE_REAL)
-        static_cast<T*>(p.out0)[off] = v.x;
+    {
+        if(p.cb.store_fn)
+            cb_store_scalar<T>(p.cb, off, v.x);
+        else
+            static_cast<T*>(p.out0)[off] = v.x;
+    }
     else
         store_elem<T, VEC>(p, off, v);
 }
@@ -524,13 +604,9 @@ FFT_DEV void real_post_elem(const fftk_real_params& p, uint64_t gid)
         o1.x *= (T)p.scale;
         o1.y *= (T)p.scale;
     }
-    h0[hb + (int64_t)j * p.h_s] = o0.x;
-    h1[hb + (int64_t)j * p.h_s] = o0.y;
+    cb_or_store<T>(p.cb, h0, h1, hb + (int64_t)j * p.h_s, o0);
     if(two)
-    {
-        h0[hb + (int64_t)jq * p.h_s] = o1.x;
-        h1[hb + (int64_t)jq * p.h_s] = o1.y;
-    }
+        cb_or_store<T>(p.cb, h0, h1, hb + (int64_t)jq * p.h_s, o1);
 }
 
 template <typename T>
@@ -554,15 +630,13 @@ FFT_DEV void real_pre_elem(const fftk_real_params& p, uint64_t gid)
     int64_t  zb = (int64_t)r0 * p.z_r0 + (int64_t)r1 * p.z_r1 + (int64_t)r2 * p.z_r2;
     int64_t  hb = (int64_t)r0 * p.h_r0 + (int64_t)r1 * p.h_r1 + (int64_t)r2 * p.h_r2;
     uint32_t jq = L - j;
-    C        a;
-    a.x = h0[hb + (int64_t)j * p.h_s];
-    a.y = h1[hb + (int64_t)j * p.h_s];
-    C    zj, zq;
-    bool two = true;
+    C        a   = cb_or_load<T>(p.cb, h0, h1, hb + (int64_t)j * p.h_s);
+    C        zj, zq;
+    bool     two = true;
     zq.x = zq.y = 0;
     if(j == 0)
     {
-        T bx = h0[hb + (int64_t)L * p.h_s];
+        T bx = cb_or_load<T>(p.cb, h0, h1, hb + (int64_t)L * p.h_s).x;
         zj.x = a.x + bx;
         zj.y = a.x - bx;
         two  = false;
@@ -575,9 +649,7 @@ FFT_DEV void real_pre_elem(const fftk_real_params& p, uint64_t gid)
     }
     else
     {
-        C b;
-        b.x  = h0[hb + (int64_t)jq * p.h_s];
-        b.y  = h1[hb + (int64_t)jq * p.h_s];
+        C b  = cb_or_load<T>(p.cb, h0, h1, hb + (int64_t)jq * p.h_s);
         C u  = c_add(a, b);
         C v  = c_sub(a, b);
         C t  = static_cast<const C*>(p.half_tw)[j];
@@ -689,8 +761,26 @@ FFT_DEV void copy_elem(const fftk_copy_params& p, uint64_t gid)
     const int64_t db   = (int64_t)r0 * p.d_r0 + (int64_t)r1 * p.d_r1 + (int64_t)r2 * p.d_r2;
     const bool    flip = p.mirror_from && j >= p.mirror_from;
     const int64_t so   = sb + (int64_t)(flip ? p.mirror_n - j : j) * p.s_s;
-    T             re   = static_cast<const T*>(p.s0)[so];
-    T             im   = p.src_real ? (T)0 : static_cast<const T*>(p.s1)[so];
+    T             re, im;
+    if(p.cb.load_fn)
+    {
+        if(p.src_real)
+        {
+            re = cb_load_scalar<T>(p.cb, so);
+            im = 0;
+        }
+        else
+        {
+            typename cplx_of<T>::type v = cb_or_load<T>(p.cb, static_cast<const T*>(p.s0), static_cast<const T*>(p.s1), so);
+            re                          = v.x;
+            im                          = v.y;
+        }
+    }
+    else
+    {
+        re = static_cast<const T*>(p.s0)[so];
+        im = p.src_real ? (T)0 : static_cast<const T*>(p.s1)[so];
+    }
     if(flip)
         im = -im;
     if(p.zero_im0 && j == 0)
@@ -701,6 +791,19 @@ FFT_DEV void copy_elem(const fftk_copy_params& p, uint64_t gid)
         im *= (T)p.scale;
     }
     const int64_t dof           = db + (int64_t)j * p.d_s;
+    if(p.cb.store_fn)
+    {
+        if(p.dst_real)
+            cb_store_scalar<T>(p.cb, dof, re);
+        else
+        {
+            typename cplx_of<T>::type v;
+            v.x = re;
+            v.y = im;
+            cb_or_store<T>(p.cb, static_cast<T*>(p.d0), static_cast<T*>(p.d1), dof, v);
+        }
+        return;
+    }
     static_cast<T*>(p.d0)[dof] = re;
     if(!p.dst_real)
         static_cast<T*>(p.d1)[dof] = im;

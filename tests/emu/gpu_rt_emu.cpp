@@ -116,8 +116,15 @@ int fftrt_device_info(int* device, int* compute_units, int* lds_bytes, char* arc
     }
     return 0;
 }
+static long g_malloc_calls = 0;
+// (tests) device allocations made so far
+__attribute__((visibility("default"))) long fftrt_emu_malloc_calls(void)
+{
+    return g_malloc_calls;
+}
 int fftrt_malloc(void** ptr, size_t bytes)
 {
+    ++g_malloc_calls;
     *ptr = malloc(bytes ? bytes : 1);
     return *ptr ? 0 : 2;
 }

@@ -75,6 +75,28 @@ def test_callbacks_through_the_emulation(emu, which):
         check_case(emu, H.HostBackend(), cblib, kind, lengths, batch, precision, kw, which)
 
 
+def test_callbacks_run_inside_the_kernels(emu):
+    """no staged copies: an execution with callbacks makes no device allocation (the plan needs
+    no work area here), and the plan's pass count does not depend on callbacks"""
+    cblib = callback_library("libcb_host.so")
+    emu.c.fftrt_emu_malloc_calls.restype = ctypes.c_long
+    for kind, lengths, batch, precision, kw in CASES:
+        if kw.get("inplace"):
+            continue
+        before = []
+
+        def hook(info, backend, rt, _inner=make_hook(cblib, kind, precision, "load+store")):
+            keep = _inner(info, backend, rt)
+            before.append(emu.c.fftrt_emu_malloc_calls())  # plan and tables exist by now
+            return keep
+
+        H.run_transform(emu, H.HostBackend(), kind, lengths, batch, precision, info_hook=hook, **kw)
+        after = emu.c.fftrt_emu_malloc_calls()
+        st, text, work = emu.describe(B.NOTINPLACE, kind, precision, lengths, batch)
+        if work == 0:
+            assert after == before[0], (kind, lengths, text)
+
+
 def test_callback_rules(emu):
     info = B.ExecutionInfo(emu)
     fn = (ctypes.c_void_p * 1)(1)
@@ -104,63 +126,63 @@ def test_callbacks_on_the_gpu(gpu_lib, which):
 
 
 @pytest.mark.gpu
-def test_staged_executions_replay_from_a_graph(gpu_lib):
-    """Executions that stage through copies (callbacks, half precision) keep their copies in
-    buffers the plan owns per stream: the first execution on a stream allocates them, later
-    ones allocate nothing and can be captured.  Every replay is checked against an eager
-    execution, with eager work between the replays."""
+def test_callbacks_and_half_precision_replay_from_a_graph(gpu_lib):
+    """Callbacks are called from inside the first and last kernel of the plan: an execution
+    with callbacks allocates nothing and can be captured into a graph straight away.  Half
+    precision stages through copies in buffers the plan owns per stream: the first execution
+    on a stream allocates them (so it cannot be the captured one), later ones allocate nothing.
+    Every replay is checked against an eager result, with eager work between the replays."""
     import torch
 
     lib = gpu_lib
     dev = torch.device("cuda:0")
     cblib = callback_library("libcb_device.so")
-    n, batch = 4096, 6
     gen = torch.Generator(device=dev).manual_seed(3)
-    x = torch.view_as_complex(torch.rand((batch, n, 2), generator=gen, device=dev) - 0.5)
     scales = torch.tensor([S_LOAD, S_STORE], dtype=torch.float32, device=dev)
-    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], batch, lib=lib)
     side = torch.cuda.Stream()
-
-    def new_info():
+    # one kernel (4096), a split into two (2^17: the callbacks sit in different kernels), and
+    # the one-workgroup kernel's length (32768: the run-time-schedule pass list takes over)
+    for n, batch in ((4096, 6), (1 << 17, 2), (32768, 3)):
+        x = torch.view_as_complex(torch.rand((batch, n, 2), generator=gen, device=dev) - 0.5)
+        plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], batch, lib=lib)
         info = B.ExecutionInfo(lib).set_stream(side.cuda_stream)
         info.set_load_callback(cblib.cb_get(0, 1, 0), scales[0:].data_ptr())
         info.set_store_callback(cblib.cb_get(1, 1, 0), scales[1:].data_ptr())
-        return info
+        wb = plan.work_buffer_size
+        if wb:
+            work = torch.empty(wb, dtype=torch.uint8, device=dev)
+            info.set_work_buffer(work.data_ptr(), wb)
+        xin = x.clone()
+        y = torch.zeros_like(x)
+        ref = torch.fft.fft(x, dim=1) * (S_LOAD * S_STORE)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                plan.execute([xin.data_ptr()], [y.data_ptr()], info)  # the first execution of this plan
+        torch.cuda.synchronize()
+        for rep in range(3):
+            xin.copy_(x * (rep + 2))
+            y.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            err = (torch.linalg.vector_norm(y - ref * (rep + 2)) / torch.linalg.vector_norm(ref)).item()
+            assert err < 1e-5 * (rep + 2), (n, rep, err)
+        assert torch.equal(xin, x * 4), n  # out of place: the input is left alone
 
-    xin = x.clone()
-    y = torch.zeros_like(x)
-    info = new_info()
+    # half precision
+    hplan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256], 4, lib=lib)
+    xh = (torch.rand((4, 256, 2), generator=gen, device=dev) - 0.5).to(torch.float16)
+    yh = torch.zeros_like(xh)
+    hinfo = B.ExecutionInfo(lib).set_stream(side.cuda_stream)
     torch.cuda.synchronize()
     # before the plan has buffers for this stream, a captured execution is refused
     g0 = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
         with torch.cuda.graph(g0, stream=side):
-            refused = plan.execute_status([xin.data_ptr()], [y.data_ptr()], info)
+            refused = hplan.execute_status([xh.data_ptr()], [yh.data_ptr()], hinfo)
     assert refused == B.STATUS_FAILURE
-    # the first eager execution on the stream allocates them
-    plan.execute([xin.data_ptr()], [y.data_ptr()], info)
-    side.synchronize()
-    ref = torch.fft.fft(x, dim=1) * (S_LOAD * S_STORE)
-    assert (torch.linalg.vector_norm(y - ref) / torch.linalg.vector_norm(ref)).item() < 1e-5
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
-        with torch.cuda.graph(g, stream=side):
-            plan.execute([xin.data_ptr()], [y.data_ptr()], info)
-    torch.cuda.synchronize()
-    for rep in range(3):
-        xin.copy_(x * (rep + 2))
-        y.zero_()
-        torch.cuda.synchronize()
-        g.replay()
-        torch.cuda.synchronize()
-        err = (torch.linalg.vector_norm(y - ref * (rep + 2)) / torch.linalg.vector_norm(ref)).item()
-        assert err < 1e-5 * (rep + 2), (rep, err)
-
-    # half precision the same way
-    hplan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256], 4, lib=lib)
-    xh = (torch.rand((4, 256, 2), generator=gen, device=dev) - 0.5).to(torch.float16)
-    yh = torch.zeros_like(xh)
-    hinfo = B.ExecutionInfo(lib).set_stream(side.cuda_stream)
     hplan.execute([xh.data_ptr()], [yh.data_ptr()], hinfo)
     side.synchronize()
     want = yh.clone()
