@@ -238,7 +238,122 @@ __device__ __forceinline__ void fk_passes(const fftk_params& p, typename cplx_of
     fk_passes_tw<T, Cfg>(p.tw, lds, w, tt, active, r, lds_busy);
 }
 
-// Lean path: both sides are interleaved complex arrays whose element offsets inside a
+// Global-memory accessors of the lean path.  A side is either an array of interleaved
+// (re, im) pairs or two arrays, one of real and one of imaginary parts (planar); offsets count
+// complex elements.  at2/put2 take a wave-uniform 64-bit part and a 32-bit lane part.
+template <typename T>
+struct FkPairsIn
+{
+    typedef typename cplx_of<T>::type C;
+    const C* p;     // element 0 of the tile
+    const C* first; // element 0 of the array
+    FFT_DEV C at(uint32_t off) const
+    {
+        return p[off];
+    }
+    FFT_DEV C at2(uint64_t a, uint32_t b) const
+    {
+        const C* pk = p + a;
+        return pk[b];
+    }
+    FFT_DEV C at_or_first(bool valid, uint32_t off) const
+    {
+        const C* pj = valid ? p + off : first;
+        return *pj;
+    }
+};
+template <typename T>
+struct FkPlanarIn
+{
+    typedef typename cplx_of<T>::type C;
+    const T *re, *im, *first_re, *first_im;
+    FFT_DEV C at(uint32_t off) const
+    {
+        C v;
+        v.x = re[off];
+        v.y = im[off];
+        return v;
+    }
+    FFT_DEV C at2(uint64_t a, uint32_t b) const
+    {
+        const T *pr = re + a, *pi = im + a;
+        C        v;
+        v.x = pr[b];
+        v.y = pi[b];
+        return v;
+    }
+    FFT_DEV C at_or_first(bool valid, uint32_t off) const
+    {
+        const T *pr = valid ? re + off : first_re, *pi = valid ? im + off : first_im;
+        C        v;
+        v.x = *pr;
+        v.y = *pi;
+        return v;
+    }
+};
+// real samples (offsets count scalars); the imaginary part reads as zero
+template <typename T>
+struct FkRealIn
+{
+    typedef typename cplx_of<T>::type C;
+    const T *re, *first_re;
+    FFT_DEV C at_or_first(bool valid, uint32_t off) const
+    {
+        const T* pr = valid ? re + off : first_re;
+        C        v;
+        v.x = *pr;
+        v.y = 0;
+        return v;
+    }
+};
+template <typename T>
+struct FkPairsOut
+{
+    typedef typename cplx_of<T>::type C;
+    C* p;
+    FFT_DEV void put(uint32_t off, C v) const
+    {
+        p[off] = v;
+    }
+    FFT_DEV void put2(uint64_t a, uint32_t b, C v) const
+    {
+        C* pk = p + a;
+        pk[b] = v;
+    }
+};
+template <typename T>
+struct FkPlanarOut
+{
+    typedef typename cplx_of<T>::type C;
+    T *re, *im;
+    FFT_DEV void put(uint32_t off, C v) const
+    {
+        re[off] = v.x;
+        im[off] = v.y;
+    }
+    FFT_DEV void put2(uint64_t a, uint32_t b, C v) const
+    {
+        T *pr = re + a, *pi = im + a;
+        pr[b] = v.x;
+        pi[b] = v.y;
+    }
+};
+
+// only the real part is written (offsets count scalars)
+template <typename T>
+struct FkRealOut
+{
+    typedef typename cplx_of<T>::type C;
+    T* re;
+    FFT_DEV void put2(uint64_t a, uint32_t b, C v) const
+    {
+        T* pr = re + a;
+        pr[b] = v.x;
+    }
+};
+
+// Lean path: both sides are complex arrays (interleaved pairs, or planar: in_planar /
+// out_planar) whose element offsets inside a
 // tile fit 32 bits.  Every address is a wave-uniform 64-bit base plus a 32-bit per-lane
 // element offset and there is no per-element branching on the operation kind, so the loads
 // of a thread issue back to back.  Covers plain passes, the large twiddle, scaling, the
@@ -275,6 +390,28 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     const uint32_t q   = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
     C              r[Cfg::EPT];
     bool           lds_busy = false;
+    const FkPairsIn<T>   in_pairs{src, reinterpret_cast<const C*>(static_cast<const T*>(p.in0))};
+    const FkPlanarIn<T>  in_planar{static_cast<const T*>(p.in0) + c.ibase, static_cast<const T*>(p.in1) + c.ibase,
+                                  static_cast<const T*>(p.in0), static_cast<const T*>(p.in1)};
+    const FkPairsOut<T>  out_pairs{dst};
+    const FkPlanarOut<T> out_planar{static_cast<T*>(p.out0) + c.obase, static_cast<T*>(p.out1) + c.obase};
+// runs body(accessor) with the accessor of the side's array kind
+#define FK_WITH_IN(body)     \
+    do                       \
+    {                        \
+        if(p.in_planar)      \
+            body(in_planar); \
+        else                 \
+            body(in_pairs);  \
+    } while(0)
+#define FK_WITH_OUT(body)     \
+    do                        \
+    {                         \
+        if(p.out_planar)      \
+            body(out_planar); \
+        else                  \
+            body(out_pairs);  \
+    } while(0)
 
     // ---------------------------------------------------------------- load
     if(p.load_op == FFTK_LOAD_C2R_PRE)
@@ -326,7 +463,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 __syncthreads();
             }
         }
-        if(ok)
+        auto pre_pairs = [&](auto in) __attribute__((always_inline))
         {
 #pragma unroll
             for(int i = 0; i < PAIR_IT; ++i)
@@ -343,8 +480,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 }
                 else
                 {
-                    a  = src[j * p.t_is_c + wo];
-                    bq = src[jq * p.t_is_c + wo];
+                    a  = in.at(j * p.t_is_c + wo);
+                    bq = in.at(jq * p.t_is_c + wo);
                 }
                 C              zj, zq;
                 if(j == 0)
@@ -367,19 +504,21 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             }
             if(N % 2 == 0 && tt == 0)
             {
-                C a = (STAGE_OK && staged) ? pm : src[(N / 2) * p.t_is_c + wo];
+                C a = (STAGE_OK && staged) ? pm : in.at((N / 2) * p.t_is_c + wo);
                 C z;
                 z.x                         = (T)2 * a.x;
                 z.y                         = (T)-2 * a.y;
                 lds[fk_addr<Cfg>(w, N / 2)] = c_swap(z);
             }
-        }
+        };
+        if(ok)
+            FK_WITH_IN(pre_pairs);
         __syncthreads();
         if(active)
             fk_read<T, Cfg, 0>(lds, w, tt, r);
         lds_busy = true;
     }
-    else if(ODD_REAL && p.load_op == FFTK_LOAD_REAL)
+    else if(ODD_REAL && p.load_op == FFTK_LOAD_REAL && !(p.flags & FFTK_F_CHIRP_LOAD))
     {
         // odd-length real forward: real samples (strides in scalars), imaginary parts zero
         const T*       srcr = static_cast<const T*>(p.in0) + c.ibase;
@@ -402,12 +541,12 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 }
         }
     }
-    else if(ODD_REAL && p.load_op == FFTK_LOAD_HERM_EXPAND)
+    else if(ODD_REAL && p.load_op == FFTK_LOAD_HERM_EXPAND && !(p.flags & FFTK_F_CHIRP_LOAD))
     {
         // odd-length real inverse: bins 0..N/2 are stored, bin j > N/2 is the conjugate of bin
         // N-j; the imaginary part of bin 0 is ignored
         const uint32_t wo = w * p.w_is_c;
-        if(ok)
+        auto expand = [&](auto in) __attribute__((always_inline))
         {
 #pragma unroll
             for(int s = 0; s < S0; ++s)
@@ -418,7 +557,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     const uint32_t jm = j <= (uint32_t)(N / 2) ? j : (uint32_t)N - j;
                     if(fk_live<Cfg, 0>(tt, s))
                     {
-                        C v = src[jm * p.t_is_c + wo];
+                        C v = in.at(jm * p.t_is_c + wo);
                         if(jm != j)
                             v.y = -v.y;
                         if(j == 0)
@@ -426,7 +565,9 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         r[s * R0 + k] = inv ? c_swap(v) : v;
                     }
                 }
-        }
+        };
+        if(ok)
+            FK_WITH_IN(expand);
     }
     else if(STAGE_OK && p.stage_io)
     {
@@ -459,22 +600,39 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 // first element of the array instead of being skipped, so that all loads stay in
                 // flight (not to the first sample of this tile: the tile itself lies beyond the
                 // array when the table-indexed axis is longer than the signal)
-                const C*   first = reinterpret_cast<const C*>(static_cast<const T*>(p.in0));
                 const C*   chirp = static_cast<const C*>(p.chirp);
                 const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
                 C          ch[Cfg::EPT];
+                const bool herm  = p.load_op == FFTK_LOAD_HERM_EXPAND;
+                auto       fetch = [&](auto in) __attribute__((always_inline))
+                {
 #pragma unroll
-                for(int s = 0; s < S0; ++s)
+                    for(int s = 0; s < S0; ++s)
 #pragma unroll
-                    for(int k = 0; k < R0; ++k)
-                    {
-                        const uint32_t j     = tt + s * Cfg::TPT + k * M0;
-                        const uint32_t idx   = j * p.chirp_js + q * p.chirp_qs;
-                        const bool     valid = idx < p.blu_n && fk_live<Cfg, 0>(tt, s);
-                        const C*       pj    = valid ? src + (j * p.t_is_c + w * p.w_is_c) : first;
-                        r[s * R0 + k]        = *pj;
-                        ch[s * R0 + k]       = chirp[valid ? idx : 0u];
-                    }
+                        for(int k = 0; k < R0; ++k)
+                        {
+                            const uint32_t j     = tt + s * Cfg::TPT + k * M0;
+                            const uint32_t idx   = j * p.chirp_js + q * p.chirp_qs;
+                            const bool     valid = idx < p.blu_n && fk_live<Cfg, 0>(tt, s);
+                            // Hermitian input of an odd-length real inverse transform (chirp index =
+                            // sample index there): bins above n_in/2 are the conjugate mirror
+                            const uint32_t jm = (herm && j > p.n_in / 2) ? p.n_in - j : j;
+                            C              v  = in.at_or_first(valid, jm * p.t_is_c + w * p.w_is_c);
+                            if(herm)
+                            {
+                                if(jm != j)
+                                    v.y = -v.y;
+                                if(j == 0 || 2 * j == p.n_in)
+                                    v.y = 0;
+                            }
+                            r[s * R0 + k]  = v;
+                            ch[s * R0 + k] = chirp[valid ? idx : 0u];
+                        }
+                };
+                if(p.load_op == FFTK_LOAD_REAL)
+                    fetch(FkRealIn<T>{static_cast<const T*>(p.in0) + c.ibase, static_cast<const T*>(p.in0)});
+                else
+                    FK_WITH_IN(fetch);
 #pragma unroll
                 for(int s = 0; s < S0; ++s)
 #pragma unroll
@@ -494,15 +652,16 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             }
             else
             {
+                auto fetch = [&](auto in) __attribute__((always_inline))
+                {
 #pragma unroll
-                for(int s = 0; s < S0; ++s)
+                    for(int s = 0; s < S0; ++s)
 #pragma unroll
-                    for(int k = 0; k < R0; ++k)
-                    {
-                        const C* pk = src + (uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c;
-                        if(fk_live<Cfg, 0>(tt, s))
-                            r[s * R0 + k] = pk[li];
-                    }
+                        for(int k = 0; k < R0; ++k)
+                            if(fk_live<Cfg, 0>(tt, s))
+                                r[s * R0 + k] = in.at2((uint64_t)(s * Cfg::TPT + k * M0) * p.t_is_c, li);
+                };
+                FK_WITH_IN(fetch);
             }
             if(inv)
             {
@@ -666,7 +825,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 return;
             }
         }
-        if(ok)
+        auto post_pairs = [&](auto out) __attribute__((always_inline))
         {
             const C*       htw = static_cast<const C*>(p.half_tw);
             const uint32_t wo  = w * p.w_os_c;
@@ -705,18 +864,20 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 o0.y *= sc;
                 o1.x *= sc;
                 o1.y *= sc;
-                dst[j * p.t_os_c + wo]  = o0;
-                dst[jq * p.t_os_c + wo] = o1;
+                out.put(j * p.t_os_c + wo, o0);
+                out.put(jq * p.t_os_c + wo, o1);
             }
             if(N % 2 == 0 && tt == 0)
             {
                 C z = lds[fk_addr<Cfg>(w, N / 2)];
                 C o;
-                o.x                            = z.x * sc;
-                o.y                            = -z.y * sc;
-                dst[(N / 2) * p.t_os_c + wo] = o;
+                o.x = z.x * sc;
+                o.y = -z.y * sc;
+                out.put((N / 2) * p.t_os_c + wo, o);
             }
-        }
+        };
+        if(ok)
+            FK_WITH_OUT(post_pairs);
         return;
     }
 
@@ -826,20 +987,24 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
                     ch[s * RL + k]     = chirp[(idx < p.blu_n && fk_live<Cfg, LAST>(ot, s)) ? idx : 0u];
                 }
+            auto emit = [&](auto out) __attribute__((always_inline))
+            {
 #pragma unroll
-            for(int s = 0; s < SL; ++s)
+                for(int s = 0; s < SL; ++s)
 #pragma unroll
-                for(int k = 0; k < RL; ++k)
-                {
-                    const uint32_t j   = ot + s * Cfg::TPT + k * CL;
-                    const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
-                    C v = cj ? c_mul(r[s * RL + k], ch[s * RL + k]) : c_mulc(r[s * RL + k], ch[s * RL + k]);
-                    if(idx < p.blu_n && j < p.n_out && fk_live<Cfg, LAST>(ot, s))
+                    for(int k = 0; k < RL; ++k)
                     {
-                        C* pk  = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
-                        pk[lo] = v;
+                        const uint32_t j   = ot + s * Cfg::TPT + k * CL;
+                        const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
+                        C v = cj ? c_mul(r[s * RL + k], ch[s * RL + k]) : c_mulc(r[s * RL + k], ch[s * RL + k]);
+                        if(idx < p.blu_n && j < p.n_out && fk_live<Cfg, LAST>(ot, s))
+                            out.put2((uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c, lo, v);
                     }
-                }
+            };
+            if(p.store_op == FFTK_STORE_REAL)
+                emit(FkRealOut<T>{static_cast<T*>(p.out0) + c.obase});
+            else
+                FK_WITH_OUT(emit);
         }
         else if(ODD_REAL && p.store_op == FFTK_STORE_REAL)
         {
@@ -857,18 +1022,23 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         }
         else
         {
+            auto emit = [&](auto out) __attribute__((always_inline))
+            {
 #pragma unroll
-            for(int s = 0; s < SL; ++s)
+                for(int s = 0; s < SL; ++s)
 #pragma unroll
-                for(int k = 0; k < RL; ++k)
-                {
-                    C* pk = dst + (uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c;
-                    // an odd-length real forward transform keeps the first n_out bins
-                    if(fk_live<Cfg, LAST>(ot, s) && (!ODD_REAL || ot + s * Cfg::TPT + k * CL < p.n_out))
-                        pk[lo] = r[s * RL + k];
-                }
+                    for(int k = 0; k < RL; ++k)
+                    {
+                        // an odd-length real forward transform keeps the first n_out bins
+                        if(fk_live<Cfg, LAST>(ot, s) && (!ODD_REAL || ot + s * Cfg::TPT + k * CL < p.n_out))
+                            out.put2((uint64_t)(s * Cfg::TPT + k * CL) * p.t_os_c, lo, r[s * RL + k]);
+                    }
+            };
+            FK_WITH_OUT(emit);
         }
     }
+#undef FK_WITH_IN
+#undef FK_WITH_OUT
 }
 
 template <typename T, typename Cfg, bool VEC, bool LEAN>

@@ -89,6 +89,8 @@ struct fftk_params
     uint32_t lean;       // fast kernel: plain interleaved complex in and out, strides below in
                          // complex elements fit 32 bits: branch-free addressing path
     uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
+    uint32_t in_planar, out_planar; // lean path: that side is a planar complex array (real parts
+                                    // at in0/out0, imaginary parts at in1/out1)
     uint32_t n2;       // fused 2D kernel: length of the second (strided) dimension; tw2: its twiddles
     uint32_t stage_io; // lean path: move the tile between global memory and LDS with consecutive
                        // lanes on consecutive elements (transforms too short for coalesced

@@ -860,13 +860,37 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     if(s.load_op == FFTK_LOAD_REAL || s.store_op == FFTK_STORE_REAL)
         vec = false;
     rec.vec_ok = vec;
-    // branch-free addressing path of the fast kernel: interleaved complex on both sides
-    // (real pairs with unit real stride count), element offsets inside a tile fit 32 bits
+    // branch-free addressing path of the fast kernel: complex arrays on both sides (real pairs
+    // with unit real stride count), element offsets inside a tile fit 32 bits.  A side is
+    // interleaved (even scalar strides) or planar (scalar strides are element strides).
+    auto even_side = [&](bool in) {
+        bool ok = in ? (even(k.t_is) && even(k.w_is)) : (even(k.t_os) && even(k.w_os));
+        for(int i = 0; i < 3; ++i)
+            ok = ok && even(in ? k.o_is[i] : k.o_os[i]);
+        return ok;
+    };
+    // 0: no lean access, 1: interleaved, 2: planar, 3: real scalars
+    auto side_kind = [&](const IoRef& io, bool real_scalar, bool in) {
+        if(io.planar)
+            return real_scalar ? 0 : 2;
+        if(real_scalar)
+            return 3;
+        return io_vec_ok(io, real_scalar) && even_side(in) ? 1 : 0;
+    };
+    int in_kind = side_kind(rec.src, s.src_real_scalar, true), out_kind = side_kind(rec.dst, s.dst_real_scalar, false);
+    // real sides: only together with the Bluestein chirp of that side (odd-length real transforms of
+    // lengths with large prime factors); the plain odd-length real kernels follow below
+    const bool chirp_rows = (k.flags & FFTK_F_CHIRP_LOAD) && k.chirp_js == 1 && k.chirp_qs == 0 && k.n_in == k.blu_n;
+    if((in_kind == 3) != (s.load_op == FFTK_LOAD_REAL) || (in_kind == 3 && !chirp_rows))
+        in_kind = 0;
+    if((out_kind == 3) != (s.store_op == FFTK_STORE_REAL) || (out_kind == 3 && !(k.flags & FFTK_F_CHIRP_STORE)))
+        out_kind = 0;
     {
         const uint32_t lean_flags = FFTK_F_TWIDDLE_STORE | FFTK_F_SCALE | FFTK_F_CHIRP_LOAD
                                     | FFTK_F_CHIRP_STORE | FFTK_F_CHIRP_CONJ | FFTK_F_CONV;
-        bool ops_ok = (s.load_op == FFTK_LOAD_COMPLEX || s.load_op == FFTK_LOAD_C2R_PRE)
-                      && (s.store_op == FFTK_STORE_COMPLEX || s.store_op == FFTK_STORE_R2C_POST)
+        bool ops_ok = (s.load_op == FFTK_LOAD_COMPLEX || s.load_op == FFTK_LOAD_C2R_PRE || in_kind == 3
+                       || (s.load_op == FFTK_LOAD_HERM_EXPAND && chirp_rows))
+                      && (s.store_op == FFTK_STORE_COMPLEX || s.store_op == FFTK_STORE_R2C_POST || out_kind == 3)
                       && (k.flags & ~lean_flags) == 0;
         // short inputs/outputs are only expressed through the chirp index test
         if(k.n_in != k.n && !((k.flags & FFTK_F_CHIRP_LOAD) && k.chirp_js == 1 && k.chirp_qs == 0
@@ -878,55 +902,57 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             ops_ok = false;
         if(s.store_op == FFTK_STORE_R2C_POST && (k.flags & (FFTK_F_CHIRP_STORE | FFTK_F_TWIDDLE_STORE)))
             ops_ok = false;
-        if(k.fast && vec && ops_ok && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
+        if(k.fast && in_kind && out_kind && ops_ok && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
         {
-            uint64_t in_span  = (uint64_t)(k.n + 1) * (uint64_t)(k.t_is / 2) + (uint64_t)W * (uint64_t)(k.w_is / 2);
-            uint64_t out_span = (uint64_t)(k.n + 1) * (uint64_t)(k.t_os / 2) + (uint64_t)W * (uint64_t)(k.w_os / 2);
+            const int64_t in_div = in_kind == 1 ? 2 : 1, out_div = out_kind == 1 ? 2 : 1;
+            uint64_t in_span  = (uint64_t)(k.n + 1) * (uint64_t)(k.t_is / in_div) + (uint64_t)W * (uint64_t)(k.w_is / in_div);
+            uint64_t out_span = (uint64_t)(k.n + 1) * (uint64_t)(k.t_os / out_div) + (uint64_t)W * (uint64_t)(k.w_os / out_div);
             if(in_span < (1ull << 28) && out_span < (1ull << 28))
             {
-                rec.lean_ok = true;
+                rec.lean_ok    = true;
+                k.in_planar    = in_kind == 2;
+                k.out_planar   = out_kind == 2;
                 // short transforms in unit-stride rows: coalesced tile copies through LDS
                 // (also the fused real pre/post-processing: rows of n+1 bins on that side)
                 const bool plain_ops = s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_COMPLEX;
                 const bool real_ops  = (s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_R2C_POST)
                                       || (s.load_op == FFTK_LOAD_C2R_PRE && s.store_op == FFTK_STORE_COMPLEX);
                 if(!column && (k.T == 1 || ((size_t)k.T * esize <= 16 && k.n < 32)) && k.t_is == 2 && k.t_os == 2
+                   && in_kind == 1 && out_kind == 1
                    && (plain_ops || real_ops) && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0 && k.n_in == k.n
                    && k.n_out == k.n)
                     k.stage_io = 1;
-                k.t_is_c    = (uint32_t)(k.t_is / 2);
-                k.t_os_c    = (uint32_t)(k.t_os / 2);
-                k.w_is_c    = (uint32_t)(k.w_is / 2);
-                k.w_os_c    = (uint32_t)(k.w_os / 2);
+                k.t_is_c    = (uint32_t)(k.t_is / in_div);
+                k.t_os_c    = (uint32_t)(k.t_os / out_div);
+                k.w_is_c    = (uint32_t)(k.w_is / in_div);
+                k.w_os_c    = (uint32_t)(k.w_os / out_div);
             }
         }
     }
 
     // odd-length real transforms on the same path: real samples in -> the first n/2+1 bins out,
     // or those bins in (mirrored to the full spectrum on load) -> real samples out.  The real
-    // side is addressed in scalars, the complex side must be interleaved with even strides.
+    // side is addressed in scalars, the complex side is interleaved with even strides or planar.
     {
         const bool fwd = s.load_op == FFTK_LOAD_REAL && s.store_op == FFTK_STORE_COMPLEX && k.n_in == k.n
                          && k.n_out == k.n / 2 + 1;
         const bool bwd = s.load_op == FFTK_LOAD_HERM_EXPAND && s.store_op == FFTK_STORE_REAL && k.n_in == k.n
                          && k.n_out == k.n;
-        auto even = [](int64_t v) { return v % 2 == 0; };
-        bool cplx_ok = fwd ? (io_vec_ok(rec.dst, false) && even(k.t_os) && even(k.w_os))
-                           : (io_vec_ok(rec.src, false) && even(k.t_is) && even(k.w_is));
-        for(int i = 0; i < 3; ++i)
-            cplx_ok = cplx_ok && (fwd ? even(k.o_os[i]) : even(k.o_is[i]));
+        const int  cplx_kind = fwd ? out_kind : in_kind;
         const bool real_ok = fwd ? !rec.src.planar : !rec.dst.planar;
-        if(k.fast && (fwd || bwd) && (k.n & 1u) && cplx_ok && real_ok && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0
+        if(k.fast && (fwd || bwd) && (k.n & 1u) && cplx_kind && real_ok && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0
            && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
         {
-            const int64_t ti = fwd ? k.t_is : k.t_is / 2, wi = fwd ? k.w_is : k.w_is / 2;
-            const int64_t to = fwd ? k.t_os / 2 : k.t_os, wo = fwd ? k.w_os / 2 : k.w_os;
+            const int64_t cdiv = cplx_kind == 2 ? 1 : 2;
+            const int64_t ti = fwd ? k.t_is : k.t_is / cdiv, wi = fwd ? k.w_is : k.w_is / cdiv;
+            const int64_t to = fwd ? k.t_os / cdiv : k.t_os, wo = fwd ? k.w_os / cdiv : k.w_os;
             uint64_t      in_span  = (uint64_t)(k.n + 1) * (uint64_t)ti + (uint64_t)W * (uint64_t)wi;
             uint64_t      out_span = (uint64_t)(k.n + 1) * (uint64_t)to + (uint64_t)W * (uint64_t)wo;
             if(in_span < (1ull << 28) && out_span < (1ull << 28))
             {
                 rec.lean_ok = true;
-                rec.lean_real = true;
+                k.in_planar = bwd && cplx_kind == 2;
+                k.out_planar = fwd && cplx_kind == 2;
                 k.t_is_c    = (uint32_t)ti;
                 k.w_is_c    = (uint32_t)wi;
                 k.t_os_c    = (uint32_t)to;
@@ -2846,7 +2872,18 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
             k.out0        = d0;
             k.out1        = d1;
             bool vec = rec.vec_ok && aligned(s0, plan.elem_bytes) && aligned(d0, plan.elem_bytes);
-            k.lean   = (rec.lean_ok && vec) ? 1 : 0;
+            k.lean   = 0;
+            if(rec.lean_ok)
+            {
+                // interleaved complex sides need the alignment of a pair, planar and real sides that
+                // of a scalar
+                const size_t in_al  = (k.in_planar || k.load_op == FFTK_LOAD_REAL) ? plan.elem_bytes / 2 : plan.elem_bytes;
+                const size_t out_al = (k.out_planar || k.store_op == FFTK_STORE_REAL) ? plan.elem_bytes / 2 : plan.elem_bytes;
+                k.lean = (aligned(s0, in_al) && aligned(d0, out_al) && (!k.in_planar || aligned(s1, in_al))
+                          && (!k.out_planar || aligned(d1, out_al)))
+                             ? 1
+                             : 0;
+            }
             const bool with_cb = cb_of(pass_index, rec.src, rec.dst, k.cb);
             if(with_cb)
             {
@@ -2855,13 +2892,6 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
                     return rocfft_status_failure;
                 k.fast = 0;
                 k.lean = 0;
-            }
-            if(rec.lean_real && !with_cb)
-            {
-                // the real side needs scalar alignment only
-                const bool in_ok  = aligned(s0, k.load_op == FFTK_LOAD_REAL ? plan.elem_bytes / 2 : plan.elem_bytes);
-                const bool out_ok = aligned(d0, k.store_op == FFTK_STORE_REAL ? plan.elem_bytes / 2 : plan.elem_bytes);
-                k.lean            = (in_ok && out_ok) ? 1 : 0;
             }
             rc = fftrt_launch_tile(&k, plan.precision, vec ? 1 : 0, rec.grid, rec.lds, stream);
         }
@@ -2941,7 +2971,7 @@ std::string ExecPlan::describe() const
               << (k.out_fast_tile ? "tile" : "fft") << " flags 0x" << std::hex << k.flags << std::dec
               << " load " << k.load_op << " store " << k.store_op << (r.vec_ok ? " vec" : " scalar");
             if(r.lean_ok)
-                o << " lean";
+                o << " lean" << (k.in_planar ? " planar_in" : "") << (k.out_planar ? " planar_out" : "");
             if(k.xcd_remap)
                 o << " xcd_ranges";
             if(k.oc0_first)

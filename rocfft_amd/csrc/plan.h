@@ -84,7 +84,6 @@ struct PassRec
     IoRef                 src, dst;
     bool                  vec_ok = false;
     bool                  lean_ok = false; // eligible for the branch-free addressing path when vec holds
-    bool                  lean_real = false; // ... with real samples on one side (odd-length real transforms)
     uint32_t              grid   = 0;
     size_t                lds    = 0;
     std::string           note;

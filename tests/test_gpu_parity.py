@@ -92,6 +92,21 @@ def test_odd_real_layouts(gpu):
         for prec in (B.SINGLE, B.DOUBLE):
             H.check(lib, be, B.REAL_FORWARD, lengths, 3, prec)
             H.check(lib, be, B.REAL_INVERSE, lengths, 3, prec)
+    # lengths with a large prime factor: the chirp-z convolution in one kernel, real samples on one side
+    for n in (17, 173, 1009, 2849):
+        for prec in (B.SINGLE, B.DOUBLE):
+            H.check(lib, be, B.REAL_FORWARD, [n], 5, prec)
+            H.check(lib, be, B.REAL_INVERSE, [n], 5, prec)
+        H.check(lib, be, B.REAL_FORWARD, [n], 4, B.SINGLE, inplace=True, scale=0.5)
+        H.check(lib, be, B.REAL_INVERSE, [n], 4, B.DOUBLE, inplace=True, scale=0.25)
+        H.check(lib, be, B.REAL_FORWARD, [n], 3, B.DOUBLE, in_strides=[3], in_dist=3 * n + 1)
+        H.check(lib, be, B.REAL_INVERSE, [n], 3, B.SINGLE, out_strides=[2], out_dist=2 * n + 3)
+        H.check(lib, be, B.REAL_FORWARD, [n], 2, B.SINGLE, in_offsets=[1, 0], out_offsets=[3, 0])
+        H.check(lib, be, B.REAL_INVERSE, [n], 2, B.SINGLE, in_offsets=[5, 0], out_offsets=[1, 0])
+    for lengths in ([173, 14, 27], [2849, 9], [97, 97]):
+        for prec in (B.SINGLE, B.DOUBLE):
+            H.check(lib, be, B.REAL_FORWARD, lengths, 3, prec)
+            H.check(lib, be, B.REAL_INVERSE, lengths, 3, prec)
 
 
 def test_compiled_schedules_in_other_layouts(gpu):
@@ -114,6 +129,46 @@ def test_compiled_schedules_in_other_layouts(gpu):
     for n in (5000, 6000, 9000, 10000, 6561, 100000):
         H.check(lib, be, K.COMPLEX_FORWARD, [n], 2, K.SINGLE)
         H.check(lib, be, K.REAL_INVERSE, [n], 2, K.DOUBLE)
+
+
+def test_planar_arrays_on_the_compiled_kernels(gpu):
+    """Planar complex and Hermitian arrays (real and imaginary parts in separate buffers) take the
+    compiled kernels like interleaved ones: every fused operation of that path (plain passes,
+    Hermitian pre/post-processing of even lengths, odd-length real transforms, the Bluestein chirp
+    on load and store, column and transposing passes of 2D/3D transforms, workgroups of 1024
+    threads), planar on one side or both, in place, strided, and with different offsets of the
+    real and the imaginary array."""
+    lib, be = gpu
+    K = B
+    CP, CI, HP = K.COMPLEX_PLANAR, K.COMPLEX_INTERLEAVED, K.HERMITIAN_PLANAR
+    st, text, _ = lib.describe(K.NOTINPLACE, K.COMPLEX_FORWARD, K.SINGLE, [1000], 8,
+                               B.PlanDescription(lib).set_data_layout(CP, CP))
+    assert st == 0 and "lean planar_in planar_out" in text and " fast" in text, text
+    for n in (6, 30, 100, 168, 243, 350, 1000, 1836, 3000, 4096, 7072, 10000):
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 5, K.SINGLE, in_type=CP, out_type=CP)
+        H.check(lib, be, K.COMPLEX_INVERSE, [n], 3, K.DOUBLE, in_type=CP, out_type=CP, inplace=True)
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 3, K.DOUBLE, in_type=CP, out_type=CI, scale=0.5)
+        H.check(lib, be, K.COMPLEX_INVERSE, [n], 3, K.SINGLE, in_type=CI, out_type=CP)
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 3, K.SINGLE, in_type=CP, out_type=CP, in_offsets=[3, 1],
+                out_offsets=[0, 5], in_strides=[2], in_dist=2 * n + 3, out_strides=[3], out_dist=3 * n)
+        # even-length real transforms: the half-length kernel with the Hermitian side planar
+        H.check(lib, be, K.REAL_FORWARD, [2 * n], 3, K.SINGLE, out_type=HP)
+        H.check(lib, be, K.REAL_INVERSE, [2 * n], 3, K.DOUBLE, in_type=HP)
+        H.check(lib, be, K.REAL_FORWARD, [2 * n], 3, K.DOUBLE, out_type=HP, out_offsets=[1, 2])
+        H.check(lib, be, K.REAL_INVERSE, [2 * n], 3, K.SINGLE, in_type=HP, in_offsets=[2, 1])
+    # odd-length real transforms, Bluestein lengths (one kernel and three kernels)
+    for n in (9, 77, 625, 1001, 4095, 173, 1009, 2849, 10007):
+        H.check(lib, be, K.REAL_FORWARD, [n], 3, K.SINGLE, out_type=HP)
+        H.check(lib, be, K.REAL_INVERSE, [n], 3, K.DOUBLE, in_type=HP)
+        H.check(lib, be, K.COMPLEX_FORWARD, [n], 3, K.DOUBLE, in_type=CP, out_type=CP)
+        H.check(lib, be, K.COMPLEX_INVERSE, [n], 3, K.SINGLE, in_type=CP, out_type=CP, inplace=True)
+    for lengths in ([100, 100], [7, 340], [91, 175], [1000, 12], [12, 1000], [360, 360], [541, 24], [64, 64],
+                    [25, 17, 135], [44, 68, 20], [9, 10, 6], [100, 77, 16], [173, 14, 27]):
+        for prec in (K.SINGLE, K.DOUBLE):
+            H.check(lib, be, K.COMPLEX_FORWARD, lengths, 2, prec, in_type=CP, out_type=CP)
+            H.check(lib, be, K.COMPLEX_INVERSE, lengths, 2, prec, in_type=CP, out_type=CP, inplace=True)
+            H.check(lib, be, K.REAL_FORWARD, lengths, 2, prec, out_type=HP)
+            H.check(lib, be, K.REAL_INVERSE, lengths, 2, prec, in_type=HP)
 
 
 @pytest.mark.parametrize("n", [16384, 32768, 65536, 2 ** 18, 2 ** 20, 6000, 30030, 10007, 4099, 8198, 65537])

@@ -193,6 +193,40 @@ def passes(text):
     return [l for l in text.splitlines() if l.strip().startswith("pass")]
 
 
+def test_planar_arrays_take_the_compiled_kernels(emu):
+    """Every pass that touches a planar array of the user still runs a compiled kernel on its
+    branch-free path, whatever the operation fused into it."""
+    CP, CI, HP, RE = B.COMPLEX_PLANAR, B.COMPLEX_INTERLEAVED, B.HERMITIAN_PLANAR, B.REAL
+
+    def described(kind, lengths, it, ot, placement=B.NOTINPLACE, prec=B.SINGLE):
+        d = B.PlanDescription(emu).set_data_layout(it, ot)
+        st, text, _ = emu.describe(placement, kind, prec, lengths, 4, d)
+        assert st == 0, (kind, lengths)
+        return passes(text)
+
+    for n in (350, 1000, 4096, 10000):
+        (p,) = described(B.COMPLEX_FORWARD, [n], CP, CP)
+        assert " lean planar_in planar_out" in p and " fast" in p, p
+        (p,) = described(B.COMPLEX_INVERSE, [n], CP, CI, prec=B.DOUBLE if n <= 4096 else B.SINGLE)
+        assert " lean planar_in " in p and "planar_out" not in p and " fast" in p, p
+        (p,) = described(B.COMPLEX_FORWARD, [n], CP, CP, placement=B.INPLACE)
+        assert " lean planar_in planar_out" in p, p
+    # even-length real: the Hermitian side of the fused pre/post-processing; odd lengths; Bluestein
+    (p,) = described(B.REAL_FORWARD, [2000], RE, HP)
+    assert " lean planar_out" in p and " fast" in p, p
+    (p,) = described(B.REAL_INVERSE, [2000], HP, RE)
+    assert " lean planar_in" in p and " fast" in p, p
+    (p,) = described(B.REAL_FORWARD, [1001], RE, HP)
+    assert " lean planar_out" in p and " fast" in p, p
+    (p,) = described(B.REAL_INVERSE, [1001], HP, RE)
+    assert " lean planar_in" in p and " fast" in p, p
+    (p,) = described(B.COMPLEX_FORWARD, [173], CP, CP)
+    assert "bluestein" in p and " lean planar_in planar_out" in p, p
+    # 2D: the row pass reads the planar input, the column pass writes the planar output
+    ps = described(B.COMPLEX_FORWARD, [360, 90], CP, CP)
+    assert all(" lean" in p and " fast" in p and "planar" in p for p in ps), ps
+
+
 def test_pass_lists_of_the_benchmark_configurations(emu):
     st, text, work = emu.describe(B.INPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4096], 1024)
     assert st == 0 and len(passes(text)) == 1 and work == 0 and "16x16x16" in text
