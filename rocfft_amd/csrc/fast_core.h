@@ -156,27 +156,56 @@ FFT_DEV void fk_write(typename cplx_of<T>::type* lds, uint32_t w, uint32_t tt,
         }
 }
 
-// tw_all: the stacked twiddle table of the schedule
+// pass 0 (no twiddles) on register data
+template <typename T, typename Cfg>
+FFT_DEV void fk_compute0(uint32_t tt, typename cplx_of<T>::type* r)
+{
+    constexpr int R = Cfg::radix(0);
+    constexpr int S = Cfg::S(0);
+#pragma unroll
+    for(int s = 0; s < S; ++s)
+        if(fk_live<Cfg, 0>(tt, s))
+            Butterfly<T, R>::run(r + s * R);
+}
+
+// The twiddles of pass P (P > 0) as registers (tw_all: the stacked twiddle table of the schedule): fk_twiddles issues the loads, fk_compute_tw uses
+// them.  Issued before the LDS exchange that precedes the pass, the loads are in flight while the
+// workgroup writes, waits at the barrier and reads (idle slots read the first entry).
+template <typename Cfg, int P>
+constexpr int fk_tw_count()
+{
+    return P > 0 && P < Cfg::NP ? Cfg::S(P) * (Cfg::radix(P) - 1) : 1;
+}
 template <typename T, typename Cfg, int P>
-FFT_DEV void fk_compute(const void* tw_all, uint32_t tt, typename cplx_of<T>::type* r)
+FFT_DEV void fk_twiddles(const void* tw_all, uint32_t tt, typename cplx_of<T>::type* t)
 {
     typedef typename cplx_of<T>::type C;
     constexpr int                     R = Cfg::radix(P);
     constexpr int                     S = Cfg::S(P);
     constexpr uint32_t                c = Cfg::cum(P);
+    const C* tw = static_cast<const C*>(tw_all) + Cfg::twoff(P);
+#pragma unroll
+    for(int s = 0; s < S; ++s)
+    {
+        const uint32_t bl = fk_live<Cfg, P>(tt, s) ? (tt + s * Cfg::TPT) % c : 0u;
+#pragma unroll
+        for(int k = 1; k < R; ++k)
+            t[s * (R - 1) + k - 1] = tw[(k - 1) * c + bl];
+    }
+}
+template <typename T, typename Cfg, int P>
+FFT_DEV void fk_compute_tw(const typename cplx_of<T>::type* t, uint32_t tt, typename cplx_of<T>::type* r)
+{
+    constexpr int R = Cfg::radix(P);
+    constexpr int S = Cfg::S(P);
 #pragma unroll
     for(int s = 0; s < S; ++s)
     {
         if(!fk_live<Cfg, P>(tt, s))
             continue;
-        if(P > 0)
-        {
-            const C* tw = static_cast<const C*>(tw_all) + Cfg::twoff(P);
-            uint32_t bl = (tt + s * Cfg::TPT) % c;
 #pragma unroll
-            for(int k = 1; k < R; ++k)
-                r[s * R + k] = c_mul(r[s * R + k], tw[(k - 1) * c + bl]);
-        }
+        for(int k = 1; k < R; ++k)
+            r[s * R + k] = c_mul(r[s * R + k], t[s * (R - 1) + k - 1]);
         Butterfly<T, R>::run(r + s * R);
     }
 }
@@ -188,11 +217,15 @@ __device__ __forceinline__ void fk_passes_tw(const void* tw_all, typename cplx_o
                                              uint32_t w, uint32_t tt, bool active,
                                              typename cplx_of<T>::type* r, bool lds_busy)
 {
+    typedef typename cplx_of<T>::type C;
 #define FK_SYNC() __syncthreads()
     if(active)
-        fk_compute<T, Cfg, 0>(tw_all, tt, r);
+        fk_compute0<T, Cfg>(tt, r);
     if constexpr(Cfg::NP > 1)
     {
+        C t1[fk_tw_count<Cfg, 1>()];
+        if(active)
+            fk_twiddles<T, Cfg, 1>(tw_all, tt, t1);
         if(lds_busy)
             FK_SYNC();
         if(active)
@@ -201,11 +234,14 @@ __device__ __forceinline__ void fk_passes_tw(const void* tw_all, typename cplx_o
         if(active)
         {
             fk_read<T, Cfg, 1, A>(lds, w, tt, r);
-            fk_compute<T, Cfg, 1>(tw_all, tt, r);
+            fk_compute_tw<T, Cfg, 1>(t1, tt, r);
         }
     }
     if constexpr(Cfg::NP > 2)
     {
+        C t2[fk_tw_count<Cfg, 2>()];
+        if(active)
+            fk_twiddles<T, Cfg, 2>(tw_all, tt, t2);
         FK_SYNC();
         if(active)
             fk_write<T, Cfg, 1, A>(lds, w, tt, r);
@@ -213,11 +249,14 @@ __device__ __forceinline__ void fk_passes_tw(const void* tw_all, typename cplx_o
         if(active)
         {
             fk_read<T, Cfg, 2, A>(lds, w, tt, r);
-            fk_compute<T, Cfg, 2>(tw_all, tt, r);
+            fk_compute_tw<T, Cfg, 2>(t2, tt, r);
         }
     }
     if constexpr(Cfg::NP > 3)
     {
+        C t3[fk_tw_count<Cfg, 3>()];
+        if(active)
+            fk_twiddles<T, Cfg, 3>(tw_all, tt, t3);
         FK_SYNC();
         if(active)
             fk_write<T, Cfg, 2, A>(lds, w, tt, r);
@@ -225,7 +264,7 @@ __device__ __forceinline__ void fk_passes_tw(const void* tw_all, typename cplx_o
         if(active)
         {
             fk_read<T, Cfg, 3, A>(lds, w, tt, r);
-            fk_compute<T, Cfg, 3>(tw_all, tt, r);
+            fk_compute_tw<T, Cfg, 3>(t3, tt, r);
         }
     }
 }
@@ -423,8 +462,19 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         const C*       htw = static_cast<const C*>(p.half_tw);
         const uint32_t wo  = w * p.w_is_c;
         bool           staged = false;
-        C              pa[STAGE_OK ? PAIR_IT : 1], pb[STAGE_OK ? PAIR_IT : 1], pm;
-        pm.x = pm.y = 0;
+        // the bins of this thread's pairs (ga: bin j, gb: bin N-j, gm: bin N/2) and their twiddles;
+        // every load is issued before the first value is used, pairs beyond the row read pair 0
+        C              ga[PAIR_IT], gb[PAIR_IT], gt[PAIR_IT], gm;
+        gm.x = gm.y = 0;
+        if(ok)
+        {
+#pragma unroll
+            for(int i = 0; i < PAIR_IT; ++i)
+            {
+                const uint32_t j = tt + i * Cfg::TPT;
+                gt[i]            = htw[(!PAIR_EXACT && j >= (uint32_t)PAIRS) ? 0u : j];
+            }
+        }
         if constexpr(STAGE_OK)
         {
             if(p.stage_io)
@@ -433,6 +483,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 // (N+1 each) into LDS, then every thread takes its pairs from there
                 staged               = true;
                 const uint32_t total = p.W * (uint32_t)(N + 1);
+                C              cp[BINS_IT];
 #pragma unroll
                 for(int i = 0; i < BINS_IT; ++i)
                 {
@@ -440,10 +491,14 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     const uint32_t w_    = e / (uint32_t)(N + 1);
                     const uint32_t j_    = e - w_ * (uint32_t)(N + 1);
                     const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
-                    C              v     = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
-                    if(valid)
-                        lds[e] = v;
+                    cp[i]                = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
                 }
+                // unconditional stores (a condition would pull each load next to its store and make
+                // the thread wait for one load after the other): the LDS allocation of such a pass
+                // covers BINS_IT * nthreads elements
+#pragma unroll
+                for(int i = 0; i < BINS_IT; ++i)
+                    lds[tid + i * p.nthreads] = cp[i];
                 __syncthreads();
                 if(ok)
                 {
@@ -454,16 +509,31 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         const uint32_t j = tt + i * Cfg::TPT;
                         if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
                             continue;
-                        pa[i] = lds[row + j];
-                        pb[i] = lds[row + (uint32_t)N - j];
+                        ga[i] = lds[row + j];
+                        gb[i] = lds[row + (uint32_t)N - j];
                     }
                     if(N % 2 == 0 && tt == 0)
-                        pm = lds[row + N / 2];
+                        gm = lds[row + N / 2];
                 }
                 __syncthreads();
             }
         }
-        auto pre_pairs = [&](auto in) __attribute__((always_inline))
+        auto fetch_pairs = [&](auto in) __attribute__((always_inline))
+        {
+#pragma unroll
+            for(int i = 0; i < PAIR_IT; ++i)
+            {
+                const uint32_t j  = tt + i * Cfg::TPT;
+                const uint32_t js = (!PAIR_EXACT && j >= (uint32_t)PAIRS) ? 0u : j;
+                ga[i]             = in.at(js * p.t_is_c + wo);
+                gb[i]             = in.at(((uint32_t)N - js) * p.t_is_c + wo);
+            }
+            if(N % 2 == 0 && tt == 0)
+                gm = in.at((N / 2) * p.t_is_c + wo);
+        };
+        if(ok && !staged)
+            FK_WITH_IN(fetch_pairs);
+        if(ok)
         {
 #pragma unroll
             for(int i = 0; i < PAIR_IT; ++i)
@@ -472,17 +542,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 const uint32_t jq = N - j;
                 if(!PAIR_EXACT && j >= (uint32_t)PAIRS)
                     continue;
-                C              a, bq;
-                if(STAGE_OK && staged)
-                {
-                    a  = pa[STAGE_OK ? i : 0];
-                    bq = pb[STAGE_OK ? i : 0];
-                }
-                else
-                {
-                    a  = in.at(j * p.t_is_c + wo);
-                    bq = in.at(jq * p.t_is_c + wo);
-                }
+                const C        a = ga[i], bq = gb[i];
                 C              zj, zq;
                 if(j == 0)
                 {
@@ -491,7 +551,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 }
                 else
                 {
-                    C t  = htw[j];
+                    C t  = gt[i];
                     C u  = c_add(a, bq);
                     C v  = c_sub(a, bq);
                     zj.x = u.x + v.x * t.y - u.y * t.x;
@@ -504,15 +564,12 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             }
             if(N % 2 == 0 && tt == 0)
             {
-                C a = (STAGE_OK && staged) ? pm : in.at((N / 2) * p.t_is_c + wo);
                 C z;
-                z.x                         = (T)2 * a.x;
-                z.y                         = (T)-2 * a.y;
+                z.x                         = (T)2 * gm.x;
+                z.y                         = (T)-2 * gm.y;
                 lds[fk_addr<Cfg>(w, N / 2)] = c_swap(z);
             }
-        };
-        if(ok)
-            FK_WITH_IN(pre_pairs);
+        }
         __syncthreads();
         if(active)
             fk_read<T, Cfg, 0>(lds, w, tt, r);
@@ -573,6 +630,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     {
         // consecutive lanes copy consecutive elements of the tile into LDS
         const uint32_t total = p.W * N;
+        // every load is issued before the first value is used
+        C cp[STAGE_IT];
 #pragma unroll
         for(int i = 0; i < STAGE_IT; ++i)
         {
@@ -580,9 +639,17 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             const uint32_t w_    = e / (uint32_t)N;
             const uint32_t j_    = e - w_ * (uint32_t)N;
             const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
-            C              v     = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
-            if(valid)
-                lds[fk_addr<Cfg>(w_, j_)] = inv ? c_swap(v) : v;
+            cp[i]                = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
+        }
+        // unconditional stores, as above: the LDS allocation covers the rows up to
+        // (STAGE_IT * nthreads - 1) / N
+#pragma unroll
+        for(int i = 0; i < STAGE_IT; ++i)
+        {
+            const uint32_t e  = tid + i * p.nthreads;
+            const uint32_t w_ = e / (uint32_t)N;
+            const uint32_t j_ = e - w_ * (uint32_t)N;
+            lds[fk_addr<Cfg>(w_, j_)] = inv ? c_swap(cp[i]) : cp[i];
         }
         __syncthreads();
         if(active)
@@ -686,18 +753,25 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             // its first pass takes (tt + s TPT + k N/R), so the spectrum stays in registers
             if(active)
             {
+                // the loads of the stored spectrum are issued together (rows beyond the tile and
+                // idle slots read its first element)
+                C sp[SL * RL];
 #pragma unroll
                 for(int s = 0; s < SL; ++s)
 #pragma unroll
                     for(int k = 0; k < RL; ++k)
                     {
                         const uint32_t j = tt + s * Cfg::TPT + k * CL;
+                        sp[s * RL + k]   = cb[(ok && fk_live<Cfg, LAST>(tt, s)) ? j : 0u];
+                    }
+#pragma unroll
+                for(int s = 0; s < SL; ++s)
+#pragma unroll
+                    for(int k = 0; k < RL; ++k)
+                    {
                         if(!fk_live<Cfg, LAST>(tt, s))
                             continue;
-                        C v = r[s * RL + k];
-                        if(ok)
-                            v = c_mul(v, cb[j]);
-                        r[s * RL + k] = c_swap(v);
+                        r[s * RL + k] = c_swap(c_mul(r[s * RL + k], sp[s * RL + k]));
                     }
             }
             fk_passes<T, Cfg>(p, lds, w, tt, active, r, Cfg::NP > 1 || lds_busy);
@@ -708,6 +782,15 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 __syncthreads();
             if(active)
             {
+                C sp[SL * RL];
+#pragma unroll
+                for(int s = 0; s < SL; ++s)
+#pragma unroll
+                    for(int k = 0; k < RL; ++k)
+                    {
+                        const uint32_t j = tt + s * Cfg::TPT + k * CL;
+                        sp[s * RL + k]   = cb[(ok && fk_live<Cfg, LAST>(tt, s)) ? j : 0u];
+                    }
 #pragma unroll
                 for(int s = 0; s < SL; ++s)
 #pragma unroll
@@ -716,10 +799,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         const uint32_t j = tt + s * Cfg::TPT + k * CL;
                         if(!fk_live<Cfg, LAST>(tt, s))
                             continue;
-                        C v = r[s * RL + k];
-                        if(ok)
-                            v = c_mul(v, cb[j]);
-                        lds[fk_addr<Cfg>(w, j)] = c_swap(v);
+                        lds[fk_addr<Cfg>(w, j)] = c_swap(c_mul(r[s * RL + k], sp[s * RL + k]));
                     }
             }
             __syncthreads();
@@ -830,6 +910,15 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             const C*       htw = static_cast<const C*>(p.half_tw);
             const uint32_t wo  = w * p.w_os_c;
             const T        sc  = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
+            // the twiddle loads of all pairs are issued before the first store (a store could
+            // alias a later load and would hold it back)
+            C gt[PAIR_IT];
+#pragma unroll
+            for(int i = 0; i < PAIR_IT; ++i)
+            {
+                const uint32_t j = tt + i * Cfg::TPT;
+                gt[i]            = htw[(!PAIR_EXACT && j >= (uint32_t)PAIRS) ? 0u : j];
+            }
 #pragma unroll
             for(int i = 0; i < PAIR_IT; ++i)
             {
@@ -849,7 +938,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 else
                 {
                     C zq = lds[fk_addr<Cfg>(w, jq)];
-                    C t  = htw[j];
+                    C t  = gt[i];
                     C u, v;
                     u.x  = (T)0.5 * (zp.x + zq.x);
                     u.y  = (T)0.5 * (zp.y + zq.y);

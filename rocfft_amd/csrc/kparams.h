@@ -65,65 +65,68 @@ struct fftk_cb
 
 struct fftk_params
 {
-    // transform
-    uint32_t n;                      // FFT length
-    uint32_t nf;                     // number of passes
-    uint32_t radix[FFTK_MAX_PASSES]; // radix of each pass
-    uint32_t cum[FFTK_MAX_PASSES];   // product of the radices before the pass
-    uint32_t cshift[FFTK_MAX_PASSES]; // log2(cum) when cum is a power of two, else 0xff
-    uint32_t twoff[FFTK_MAX_PASSES]; // offset of the pass in the stacked twiddle table
-    // work split
-    uint32_t T;        // threads per transform
-    uint32_t W;        // transforms per workgroup (power of two)
-    uint32_t wshift;   // log2(W)
-    uint32_t pitch;    // LDS elements between transforms of a tile
-    uint32_t padshift; // LDS index i is stored at i + (i >> padshift)
-    uint32_t wfast;    // compute phase: 1 = neighbouring lanes take neighbouring transforms
-    uint32_t nthreads;
-    uint32_t grid;       // number of workgroups
-    uint32_t xcd_remap;  // renumber workgroups so that each XCD gets a contiguous range of tiles
-    uint32_t oc0_first;  // outer axis 0 runs faster than the tile index in the workgroup numbering
-    uint32_t fast;       // 1 = a kernel with this exact pass schedule is compiled in: use it
-    uint32_t direct_in;  // fast kernel: first pass loads global memory straight into registers
-    uint32_t direct_out; // fast kernel: last pass stores straight from registers
-    uint32_t lean;       // fast kernel: plain interleaved complex in and out, strides below in
-                         // complex elements fit 32 bits: branch-free addressing path
-    uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
-    uint32_t in_planar, out_planar; // lean path: that side is a planar complex array (real parts
-                                    // at in0/out0, imaginary parts at in1/out1)
-    uint32_t n2;       // fused 2D kernel: length of the second (strided) dimension; tw2: its twiddles
-    uint32_t stage_io; // lean path: move the tile between global memory and LDS with consecutive
-                       // lanes on consecutive elements (transforms too short for coalesced
-                       // register loads)
-    uint32_t flags;
-    int32_t  dir; // -1 forward, +1 inverse
-    uint32_t load_op, store_op;
-    uint32_t n_in;  // input elements j >= n_in read as zero
-    uint32_t n_out; // output elements j >= n_out are not written
-    uint32_t in_fast_tile, out_fast_tile; // global access runs fastest along the tile dimension
-    // index space: transform, tile dimension, three outer dimensions; strides in scalars
-    uint32_t tile_cnt;
-    uint32_t oc[3];
-    int64_t  t_is, t_os, w_is, w_os, o_is[3], o_os[3];
+    // The members the compiled kernels read on every path come first and close together: a
+    // kernel fetches its arguments from memory 64 bytes at a time, and a workgroup that runs
+    // alone (a small transform) waits for each such fetch.
     // buffers (filled in at execute)
     const void* in0;
     const void* in1;
     void*       out0;
     void*       out1;
-    // tables
-    const void* tw;        // stacked per-pass twiddles
-    const void* tw2; // fused 2D kernel: stacked twiddles of the second dimension
+    const void* tw; // stacked per-pass twiddles
+    uint32_t flags;
+    int32_t  dir; // -1 forward, +1 inverse
+    uint32_t load_op, store_op;
+    // work split
+    uint32_t W;        // transforms per workgroup (power of two)
+    uint32_t wshift;   // log2(W)
+    uint32_t wfast;    // compute phase: 1 = neighbouring lanes take neighbouring transforms
+    uint32_t nthreads;
+    uint32_t grid;       // number of workgroups
+    uint32_t xcd_remap;  // renumber workgroups so that each XCD gets a contiguous range of tiles
+    uint32_t oc0_first;  // outer axis 0 runs faster than the tile index in the workgroup numbering
+    uint32_t direct_in;  // fast kernel: first pass loads global memory straight into registers
+    uint32_t direct_out; // fast kernel: last pass stores straight from registers
+    uint32_t stage_io; // lean path: move the tile between global memory and LDS with consecutive
+                       // lanes on consecutive elements (transforms too short for coalesced
+                       // register loads)
+    uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
+    uint32_t in_planar, out_planar; // lean path: that side is a planar complex array (real parts
+                                    // at in0/out0, imaginary parts at in1/out1)
+    // index space: transform, tile dimension, three outer dimensions; strides in scalars
+    uint32_t tile_cnt;
+    uint32_t oc[3];
+    uint32_t aux_dim;   // which index is q: 0 none, 1 tile, 2/3/4 outer 0/1/2
+    uint32_t aux_shift; // aux_dim 1: q = tile index >> aux_shift (a faster plain axis was merged into the tile axis)
+    int64_t  w_is, w_os, o_is[3], o_os[3], t_is, t_os;
+    double   scale;
+    uint32_t n_in;  // input elements j >= n_in read as zero
+    uint32_t n_out; // output elements j >= n_out are not written
+    // tables of the fused operations
     const void* ltw;       // two-level table for W_L^u: lo[0 .. 1<<ltw_shift), then hi[]
-    uint32_t    ltw_shift; //
-    uint32_t    aux_dim;   // which index is q: 0 none, 1 tile, 2/3/4 outer 0/1/2
-    uint32_t    aux_shift; // aux_dim 1: q = tile index >> aux_shift (a faster plain axis was merged into the tile axis)
     const void* half_tw;   // e^{-2 pi i j/(2n)}, j in [0, n/2], for the real pre/post steps
     const void* chirp;     // Bluestein chirp e^{+i pi m^2/N}, m in [0, blu_n)
+    const void* convb;     // spectrum the tile is multiplied with in CONV mode
+    const void* tw2;       // fused 2D kernel: stacked twiddles of the second dimension
+    uint32_t    ltw_shift; //
     uint32_t    blu_n;
     uint32_t    chirp_js, chirp_qs; // logical sample index = j*chirp_js + q*chirp_qs
-    const void* convb;              // spectrum the tile is multiplied with in CONV mode
-    uint32_t    convb_qs;           // its index = j + q*convb_qs
-    double      scale;
+    uint32_t    convb_qs;           // convb index = j + q*convb_qs
+    uint32_t    n2;    // fused 2D kernel: length of the second (strided) dimension
+    uint32_t    fast;  // 1 = a kernel with this exact pass schedule is compiled in: use it
+    uint32_t    lean;  // fast kernel: complex arrays on both sides, strides in
+                       // complex elements fit 32 bits: branch-free addressing path
+    // transform: the schedule of the run-time-schedule kernel
+    uint32_t n;                      // FFT length
+    uint32_t nf;                     // number of passes
+    uint32_t T;        // threads per transform
+    uint32_t pitch;    // LDS elements between transforms of a tile
+    uint32_t padshift; // LDS index i is stored at i + (i >> padshift)
+    uint32_t in_fast_tile, out_fast_tile; // global access runs fastest along the tile dimension
+    uint32_t radix[FFTK_MAX_PASSES]; // radix of each pass
+    uint32_t cum[FFTK_MAX_PASSES];   // product of the radices before the pass
+    uint32_t cshift[FFTK_MAX_PASSES]; // log2(cum) when cum is a power of two, else 0xff
+    uint32_t twoff[FFTK_MAX_PASSES]; // offset of the pass in the stacked twiddle table
     struct fftk_cb cb; // run-time-schedule kernel only
 };
 

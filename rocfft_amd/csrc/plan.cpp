@@ -921,7 +921,14 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
                    && in_kind == 1 && out_kind == 1
                    && (plain_ops || real_ops) && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0 && k.n_in == k.n
                    && k.n_out == k.n)
+                {
                     k.stage_io = 1;
+                    // the tile copy writes LDS without bounds tests: room for every element index
+                    // its threads reach (rows of n, or of n + 1 bins on a Hermitian side)
+                    const uint64_t it_plain = (k.n + k.T - 1) / k.T, it_bins = (k.n + 1 + k.T - 1) / k.T;
+                    const uint64_t rows     = (it_plain * k.nthreads - 1) / k.n + 1;
+                    rec.lds = std::max<size_t>(rec.lds, std::max<uint64_t>(rows * k.pitch, it_bins * k.nthreads) * esize);
+                }
                 k.t_is_c    = (uint32_t)(k.t_is / in_div);
                 k.t_os_c    = (uint32_t)(k.t_os / out_div);
                 k.w_is_c    = (uint32_t)(k.w_is / in_div);
