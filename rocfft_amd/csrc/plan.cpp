@@ -869,6 +869,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             ok = ok && even(in ? k.o_is[i] : k.o_os[i]);
         return ok;
     };
+    // element offsets inside a tile are 32-bit: their byte offsets must be too
+    const uint64_t lean_span_limit = (1ull << 32) / esize;
     // 0: no lean access, 1: interleaved, 2: planar, 3: real scalars
     auto side_kind = [&](const IoRef& io, bool real_scalar, bool in) {
         if(io.planar)
@@ -907,7 +909,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             const int64_t in_div = in_kind == 1 ? 2 : 1, out_div = out_kind == 1 ? 2 : 1;
             uint64_t in_span  = (uint64_t)(k.n + 1) * (uint64_t)(k.t_is / in_div) + (uint64_t)W * (uint64_t)(k.w_is / in_div);
             uint64_t out_span = (uint64_t)(k.n + 1) * (uint64_t)(k.t_os / out_div) + (uint64_t)W * (uint64_t)(k.w_os / out_div);
-            if(in_span < (1ull << 28) && out_span < (1ull << 28))
+            if(in_span < lean_span_limit && out_span < lean_span_limit)
             {
                 rec.lean_ok    = true;
                 k.in_planar    = in_kind == 2;
@@ -955,7 +957,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             const int64_t to = fwd ? k.t_os / cdiv : k.t_os, wo = fwd ? k.w_os / cdiv : k.w_os;
             uint64_t      in_span  = (uint64_t)(k.n + 1) * (uint64_t)ti + (uint64_t)W * (uint64_t)wi;
             uint64_t      out_span = (uint64_t)(k.n + 1) * (uint64_t)to + (uint64_t)W * (uint64_t)wo;
-            if(in_span < (1ull << 28) && out_span < (1ull << 28))
+            if(in_span < lean_span_limit && out_span < lean_span_limit)
             {
                 rec.lean_ok = true;
                 k.in_planar = bwd && cplx_kind == 2;

@@ -171,6 +171,36 @@ def test_planar_arrays_on_the_compiled_kernels(gpu):
             H.check(lib, be, K.REAL_INVERSE, lengths, 2, prec, in_type=HP)
 
 
+def test_column_tiles_that_span_more_than_two_gib(gpu):
+    """A column pass whose tile reaches from the first to the last byte of a 2 GiB array: element
+    offsets inside the tile need 29 bits in single precision (129 x 2^21 elements), byte offsets 32."""
+    lib, be = gpu
+    torch = be.torch
+    n, cols = 128, 1 << 21
+    st, text, _ = lib.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], cols,
+                               B.PlanDescription(lib).set_data_layout(B.COMPLEX_INTERLEAVED, B.COMPLEX_INTERLEAVED, None,
+                                                                      None, [cols], 1, [cols], 1))
+    assert st == 0 and " lean" in text and " fast" in text, text
+    gen = torch.Generator(device=be.dev)
+    gen.manual_seed(5)
+    x = torch.view_as_complex(torch.rand((n, cols, 2), dtype=torch.float32, device=be.dev, generator=gen) - 0.5)
+    y = torch.zeros_like(x)
+    d = B.PlanDescription(lib).set_data_layout(B.COMPLEX_INTERLEAVED, B.COMPLEX_INTERLEAVED, None, None, [cols], 1,
+                                               [cols], 1)
+    plan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [n], cols, d, lib=lib)
+    plan.execute([x.data_ptr()], [y.data_ptr()])
+    torch.cuda.synchronize()
+    # the checker on three groups of columns: the first, the last and some in the middle
+    for lo in (0, cols // 2 - 77, cols - 256):
+        xs = x[:, lo:lo + 256].cpu().numpy().astype(np.complex128)
+        ref = orc.transform(B.COMPLEX_FORWARD, [n], 256, np.ascontiguousarray(xs.T), ld=False).reshape(256, n).T
+        l2, linf = orc.rel_norms(y[:, lo:lo + 256].cpu().numpy().astype(np.complex128).reshape(-1), ref.reshape(-1))
+        assert l2 <= 1e-5 and linf <= 1e-5, (lo, l2, linf)
+    # every column was written
+    assert int((y == 0).sum()) == 0
+    plan.destroy()
+
+
 @pytest.mark.parametrize("n", [16384, 32768, 65536, 2 ** 18, 2 ** 20, 6000, 30030, 10007, 4099, 8198, 65537])
 def test_long_1d(gpu, n):
     lib, be = gpu
