@@ -391,6 +391,24 @@ struct FkRealOut
     }
 };
 
+// element offset of tile entry w of the workgroup (lean path: 32-bit, strides in elements)
+template <typename T>
+FFT_DEV uint32_t fk_w_in(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
+{
+    if(!p.w_inner)
+        return w * p.w_is_c;
+    const uint32_t g = c.tile0 + w, b = g / p.w_inner;
+    return (b - c.b0) * p.w2_is_c + (g - b * p.w_inner) * p.w_is_c;
+}
+template <typename T>
+FFT_DEV uint32_t fk_w_out(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
+{
+    if(!p.w_inner)
+        return w * p.w_os_c;
+    const uint32_t g = c.tile0 + w, b = g / p.w_inner;
+    return (b - c.b0) * p.w2_os_c + (g - b * p.w_inner) * p.w_os_c;
+}
+
 // Lean path: both sides are complex arrays (interleaved pairs, or planar: in_planar /
 // out_planar) whose element offsets inside a
 // tile fit 32 bits.  Every address is a wave-uniform 64-bit base plus a 32-bit per-lane
@@ -460,7 +478,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         // writes z_j and z_{N-j} to LDS in natural order; pass 0 then reads from LDS.  An even N
         // has the unpaired bin N/2 besides.
         const C*       htw = static_cast<const C*>(p.half_tw);
-        const uint32_t wo  = w * p.w_is_c;
+        const uint32_t wo  = fk_w_in<T>(p, c, w);
         bool           staged = false;
         // the bins of this thread's pairs (ga: bin j, gb: bin N-j, gm: bin N/2) and their twiddles;
         // every load is issued before the first value is used, pairs beyond the row read pair 0
@@ -579,7 +597,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     {
         // odd-length real forward: real samples (strides in scalars), imaginary parts zero
         const T*       srcr = static_cast<const T*>(p.in0) + c.ibase;
-        const uint32_t li   = tt * p.t_is_c + w * p.w_is_c;
+        const uint32_t li   = tt * p.t_is_c + fk_w_in<T>(p, c, w);
         if(ok)
         {
 #pragma unroll
@@ -602,7 +620,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     {
         // odd-length real inverse: bins 0..N/2 are stored, bin j > N/2 is the conjugate of bin
         // N-j; the imaginary part of bin 0 is ignored
-        const uint32_t wo = w * p.w_is_c;
+        const uint32_t wo = fk_w_in<T>(p, c, w);
         auto expand = [&](auto in) __attribute__((always_inline))
         {
 #pragma unroll
@@ -658,7 +676,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     }
     else
     {
-        const uint32_t li = tt * p.t_is_c + w * p.w_is_c;
+        const uint32_t li = tt * p.t_is_c + fk_w_in<T>(p, c, w);
         if(ok)
         {
             if(p.flags & FFTK_F_CHIRP_LOAD)
@@ -671,6 +689,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
                 C          ch[Cfg::EPT];
                 const bool herm  = p.load_op == FFTK_LOAD_HERM_EXPAND;
+                const uint32_t win = fk_w_in<T>(p, c, w);
                 auto       fetch = [&](auto in) __attribute__((always_inline))
                 {
 #pragma unroll
@@ -684,7 +703,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                             // Hermitian input of an odd-length real inverse transform (chirp index =
                             // sample index there): bins above n_in/2 are the conjugate mirror
                             const uint32_t jm = (herm && j > p.n_in / 2) ? p.n_in - j : j;
-                            C              v  = in.at_or_first(valid, jm * p.t_is_c + w * p.w_is_c);
+                            C              v  = in.at_or_first(valid, jm * p.t_is_c + win);
                             if(herm)
                             {
                                 if(jm != j)
@@ -908,7 +927,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         auto post_pairs = [&](auto out) __attribute__((always_inline))
         {
             const C*       htw = static_cast<const C*>(p.half_tw);
-            const uint32_t wo  = w * p.w_os_c;
+            const uint32_t wo  = fk_w_out<T>(p, c, w);
             const T        sc  = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
             // the twiddle loads of all pairs are issued before the first store (a store could
             // alias a later load and would hold it back)
@@ -1033,7 +1052,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         }
     }
     const uint32_t oq = p.aux_dim == 1 ? (c.tile0 + ow) >> p.aux_shift : c.q_block;
-    const uint32_t lo = ot * p.t_os_c + ow * p.w_os_c;
+    const uint32_t lo = ot * p.t_os_c + fk_w_out<T>(p, c, ow);
     if(ook)
     {
         if(out_inv)

@@ -93,12 +93,18 @@ struct fftk_params
     uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
     uint32_t in_planar, out_planar; // lean path: that side is a planar complex array (real parts
                                     // at in0/out0, imaginary parts at in1/out1)
+    // Folded tile axis (w_inner != 0): tile index g counts (i, b) pairs, i = g % w_inner along the
+    // short contiguous axis (strides w_is / w_os) and b = g / w_inner along a second axis (strides
+    // w2_is / w2_os: the transforms of a batch).  A column pass over very short rows then still
+    // fills its workgroups.  tile_cnt is the number of pairs.
+    uint32_t w_inner;
+    uint32_t w2_is_c, w2_os_c; // lean path: w2_is / w2_os in elements
     // index space: transform, tile dimension, three outer dimensions; strides in scalars
     uint32_t tile_cnt;
     uint32_t oc[3];
     uint32_t aux_dim;   // which index is q: 0 none, 1 tile, 2/3/4 outer 0/1/2
     uint32_t aux_shift; // aux_dim 1: q = tile index >> aux_shift (a faster plain axis was merged into the tile axis)
-    int64_t  w_is, w_os, o_is[3], o_os[3], t_is, t_os;
+    int64_t  w_is, w_os, o_is[3], o_os[3], t_is, t_os, w2_is, w2_os;
     double   scale;
     uint32_t n_in;  // input elements j >= n_in read as zero
     uint32_t n_out; // output elements j >= n_out are not written

@@ -42,6 +42,7 @@ static bool use_fast_kernels()
 // ROCFFT_AMD_NO_XCD_REMAP=1 keeps the hardware's round-robin workgroup order (A/B comparisons)
 static const bool g_xcd_remap = !getenv("ROCFFT_AMD_NO_XCD_REMAP");
 static const bool g_share_first = !getenv("ROCFFT_AMD_NO_SHARE_FIRST");
+static const bool g_fold_tiles = !getenv("ROCFFT_AMD_NO_FOLD");
 
 struct PlanError : std::runtime_error
 {
@@ -709,6 +710,26 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     k.out_fast_tile = (tile_axis.cnt > 1 && tile_axis.os < s.t_os) ? 1 : 0;
     k.aux_dim       = tile_axis.aux ? 1 : 0;
     k.aux_shift     = tile_axis.aux ? tile_axis.aux_shift : 0;
+    // A column pass over very short rows (a 4 x 5 transform: 4 columns) would leave most lanes of
+    // its workgroups idle.  Fold the longest other plain axis (the transforms of a batch) into the
+    // tile axis: tile entries are then (column, batch item) pairs.
+    if(g_fold_tiles && (k.in_fast_tile || k.out_fast_tile) && !tile_axis.aux && tile_axis.cnt < 64 && tile_axis.is >= 0
+       && tile_axis.os >= 0)
+    {
+        int fold = -1;
+        for(size_t i = 0; i < ax.size(); ++i)
+            if(!ax[i].aux && ax[i].cnt > 1 && ax[i].is >= 0 && ax[i].os >= 0
+               && (fold < 0 || ax[i].cnt > ax[(size_t)fold].cnt))
+                fold = (int)i;
+        if(fold >= 0 && (uint64_t)tile_axis.cnt * ax[(size_t)fold].cnt < (1ull << 31))
+        {
+            k.w_inner  = tile_axis.cnt;
+            k.w2_is    = ax[(size_t)fold].is;
+            k.w2_os    = ax[(size_t)fold].os;
+            k.tile_cnt = tile_axis.cnt * ax[(size_t)fold].cnt;
+            ax.erase(ax.begin() + fold);
+        }
+    }
     for(int i = 0; i < 3; ++i)
     {
         k.oc[i]   = 1;
@@ -854,7 +875,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     // one access per (re, im) pair needs interleaved data with even scalar strides
     bool vec = io_vec_ok(rec.src, s.src_real_scalar) && io_vec_ok(rec.dst, s.dst_real_scalar);
     auto even = [](int64_t v) { return v % 2 == 0; };
-    vec = vec && even(k.t_is) && even(k.t_os) && even(k.w_is) && even(k.w_os);
+    vec = vec && even(k.t_is) && even(k.t_os) && even(k.w_is) && even(k.w_os) && even(k.w2_is) && even(k.w2_os);
     for(int i = 0; i < 3; ++i)
         vec = vec && even(k.o_is[i]) && even(k.o_os[i]);
     if(s.load_op == FFTK_LOAD_REAL || s.store_op == FFTK_STORE_REAL)
@@ -864,10 +885,16 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     // with unit real stride count), element offsets inside a tile fit 32 bits.  A side is
     // interleaved (even scalar strides) or planar (scalar strides are element strides).
     auto even_side = [&](bool in) {
-        bool ok = in ? (even(k.t_is) && even(k.w_is)) : (even(k.t_os) && even(k.w_os));
+        bool ok = in ? (even(k.t_is) && even(k.w_is) && even(k.w2_is)) : (even(k.t_os) && even(k.w_os) && even(k.w2_os));
         for(int i = 0; i < 3; ++i)
             ok = ok && even(in ? k.o_is[i] : k.o_os[i]);
         return ok;
+    };
+    // largest offset of a tile entry from the tile's base, for strides w (and w2 of a folded axis)
+    auto tile_extent = [&](int64_t w, int64_t w2) -> uint64_t {
+        if(!k.w_inner)
+            return (uint64_t)W * (uint64_t)w;
+        return ((uint64_t)(W + k.w_inner - 1) / k.w_inner + 1) * (uint64_t)w2 + (uint64_t)k.w_inner * (uint64_t)w;
     };
     // element offsets inside a tile are 32-bit: their byte offsets must be too
     const uint64_t lean_span_limit = (1ull << 32) / esize;
@@ -907,8 +934,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
         if(k.fast && in_kind && out_kind && ops_ok && k.t_is >= 0 && k.t_os >= 0 && k.w_is >= 0 && k.w_os >= 0)
         {
             const int64_t in_div = in_kind == 1 ? 2 : 1, out_div = out_kind == 1 ? 2 : 1;
-            uint64_t in_span  = (uint64_t)(k.n + 1) * (uint64_t)(k.t_is / in_div) + (uint64_t)W * (uint64_t)(k.w_is / in_div);
-            uint64_t out_span = (uint64_t)(k.n + 1) * (uint64_t)(k.t_os / out_div) + (uint64_t)W * (uint64_t)(k.w_os / out_div);
+            uint64_t in_span  = (uint64_t)(k.n + 1) * (uint64_t)(k.t_is / in_div) + tile_extent(k.w_is / in_div, k.w2_is / in_div);
+            uint64_t out_span = (uint64_t)(k.n + 1) * (uint64_t)(k.t_os / out_div) + tile_extent(k.w_os / out_div, k.w2_os / out_div);
             if(in_span < lean_span_limit && out_span < lean_span_limit)
             {
                 rec.lean_ok    = true;
@@ -935,6 +962,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
                 k.t_os_c    = (uint32_t)(k.t_os / out_div);
                 k.w_is_c    = (uint32_t)(k.w_is / in_div);
                 k.w_os_c    = (uint32_t)(k.w_os / out_div);
+                k.w2_is_c   = (uint32_t)(k.w2_is / in_div);
+                k.w2_os_c   = (uint32_t)(k.w2_os / out_div);
             }
         }
     }
@@ -955,8 +984,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
             const int64_t cdiv = cplx_kind == 2 ? 1 : 2;
             const int64_t ti = fwd ? k.t_is : k.t_is / cdiv, wi = fwd ? k.w_is : k.w_is / cdiv;
             const int64_t to = fwd ? k.t_os / cdiv : k.t_os, wo = fwd ? k.w_os / cdiv : k.w_os;
-            uint64_t      in_span  = (uint64_t)(k.n + 1) * (uint64_t)ti + (uint64_t)W * (uint64_t)wi;
-            uint64_t      out_span = (uint64_t)(k.n + 1) * (uint64_t)to + (uint64_t)W * (uint64_t)wo;
+            uint64_t      in_span  = (uint64_t)(k.n + 1) * (uint64_t)ti + tile_extent(wi, fwd ? k.w2_is : k.w2_is / cdiv);
+            uint64_t      out_span = (uint64_t)(k.n + 1) * (uint64_t)to + tile_extent(wo, fwd ? k.w2_os / cdiv : k.w2_os);
             if(in_span < lean_span_limit && out_span < lean_span_limit)
             {
                 rec.lean_ok = true;
@@ -966,6 +995,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
                 k.w_is_c    = (uint32_t)wi;
                 k.t_os_c    = (uint32_t)to;
                 k.w_os_c    = (uint32_t)wo;
+                k.w2_is_c   = (uint32_t)(fwd ? k.w2_is : k.w2_is / cdiv);
+                k.w2_os_c   = (uint32_t)(fwd ? k.w2_os / cdiv : k.w2_os);
             }
         }
     }
@@ -2985,6 +3016,8 @@ std::string ExecPlan::describe() const
                 o << " xcd_ranges";
             if(k.oc0_first)
                 o << " batch_first";
+            if(k.w_inner)
+                o << " folded(" << k.w_inner << ")";
             if(k.fast)
                 o << " fast" << (k.direct_in ? " direct_in" : " staged_in")
                   << (k.direct_out ? " direct_out" : " staged_out") << (k.stage_io ? " tile_copy" : "");

@@ -28,7 +28,26 @@ struct TileCtx
     int64_t  ibase;    // input scalar offset of (j=0, w=0)
     int64_t  obase;    // output scalar offset of (j=0, w=0)
     uint32_t q_block;  // auxiliary index when it is uniform over the workgroup
+    uint32_t b0;       // folded tile axis: second-axis index of the workgroup's first tile entry
 };
+
+// scalar offset of tile entry w of the workgroup from ibase / obase
+template <typename T>
+FFT_DEV int64_t tile_w_in(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
+{
+    if(!p.w_inner)
+        return (int64_t)w * p.w_is;
+    const uint32_t g = c.tile0 + w, b = g / p.w_inner;
+    return (int64_t)(b - c.b0) * p.w2_is + (int64_t)(g - b * p.w_inner) * p.w_is;
+}
+template <typename T>
+FFT_DEV int64_t tile_w_out(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
+{
+    if(!p.w_inner)
+        return (int64_t)w * p.w_os;
+    const uint32_t g = c.tile0 + w, b = g / p.w_inner;
+    return (int64_t)(b - c.b0) * p.w2_os + (int64_t)(g - b * p.w_inner) * p.w_os;
+}
 
 template <typename T>
 FFT_DEV void tile_decode(const fftk_params& p, uint32_t bid, TileCtx<T>& c)
@@ -63,10 +82,12 @@ FFT_DEV void tile_decode(const fftk_params& p, uint32_t bid, TileCtx<T>& c)
     c.oi[1] = bid % p.oc[1];
     c.oi[2] = bid / p.oc[1];
     c.tile0 = tb << p.wshift;
-    c.ibase = (int64_t)c.tile0 * p.w_is + (int64_t)c.oi[0] * p.o_is[0] + (int64_t)c.oi[1] * p.o_is[1]
-              + (int64_t)c.oi[2] * p.o_is[2];
-    c.obase = (int64_t)c.tile0 * p.w_os + (int64_t)c.oi[0] * p.o_os[0] + (int64_t)c.oi[1] * p.o_os[1]
-              + (int64_t)c.oi[2] * p.o_os[2];
+    c.b0    = p.w_inner ? c.tile0 / p.w_inner : 0;
+    // folded tile axis: the bases point at entry (0, b0), the per-entry offsets count from there
+    c.ibase = (p.w_inner ? (int64_t)c.b0 * p.w2_is : (int64_t)c.tile0 * p.w_is) + (int64_t)c.oi[0] * p.o_is[0]
+              + (int64_t)c.oi[1] * p.o_is[1] + (int64_t)c.oi[2] * p.o_is[2];
+    c.obase = (p.w_inner ? (int64_t)c.b0 * p.w2_os : (int64_t)c.tile0 * p.w_os) + (int64_t)c.oi[0] * p.o_os[0]
+              + (int64_t)c.oi[1] * p.o_os[1] + (int64_t)c.oi[2] * p.o_os[2];
     // (no indexing of oi[] with a run-time value: that would push the context into scratch memory)
     c.q_block = (p.aux_dim == 2 ? c.oi[0] : p.aux_dim == 3 ? c.oi[1] : p.aux_dim == 4 ? c.oi[2] : 0) >> p.aux_shift;
 }
@@ -228,7 +249,7 @@ FFT_DEV typename cplx_of<T>::type
     }
     if(ok)
     {
-        int64_t base = c.ibase + (int64_t)w * p.w_is;
+        int64_t base = c.ibase + tile_w_in<T>(p, c, w);
         if(p.load_op == FFTK_LOAD_REAL)
             v.x = p.cb.load_fn ? cb_load_scalar<T>(p.cb, base + (int64_t)j * p.t_is)
                                : static_cast<const T*>(p.in0)[base + (int64_t)j * p.t_is];
@@ -274,7 +295,7 @@ FFT_DEV void tile_load(const fftk_params&           p,
         const uint32_t n = p.n;
         tile_walk(p, tid, n / 2 + 1, p.in_fast_tile != 0, [&](uint32_t w, uint32_t j) {
             bool    ok   = c.tile0 + w < p.tile_cnt;
-            int64_t base = c.ibase + (int64_t)w * p.w_is;
+            int64_t base = c.ibase + tile_w_in<T>(p, c, w);
             C       zj, zq;
             zj.x = zj.y = zq.x = zq.y = 0;
             uint32_t jq              = n - j;
@@ -460,7 +481,7 @@ FFT_DEV void emit_elem(const fftk_params& p, const TileCtx<T>& c, uint32_t w, ui
         v.x *= (T)p.scale;
         v.y *= (T)p.scale;
     }
-    int64_t off = c.obase + (int64_t)j * p.t_os + (int64_t)w * p.w_os;
+    int64_t off = c.obase + (int64_t)j * p.t_os + tile_w_out<T>(p, c, w);
     if(p.store_op == FFTK_STORE_REAL)
     {
         if(p.cb.store_fn)
@@ -492,7 +513,7 @@ FFT_DEV void tile_store(const fftk_params&               p,
         tile_walk(p, tid, n / 2 + 1, p.out_fast_tile != 0, [&](uint32_t w, uint32_t j) {
             if(c.tile0 + w >= p.tile_cnt)
                 return;
-            int64_t  base = c.obase + (int64_t)w * p.w_os;
+            int64_t  base = c.obase + tile_w_out<T>(p, c, w);
             uint32_t jq   = n - j;
             C        zp   = lds[lds_addr(p, w, j)];
             C        o0, o1;

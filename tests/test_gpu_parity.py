@@ -171,6 +171,35 @@ def test_planar_arrays_on_the_compiled_kernels(gpu):
             H.check(lib, be, K.REAL_INVERSE, lengths, 2, prec, in_type=HP)
 
 
+def test_short_rows_with_a_batch_fold_into_full_tiles(gpu):
+    """Column passes over rows of a few elements take (column, batch item) pairs as tile entries,
+    so that small multi-dimensional transforms in a large batch fill their workgroups: all four
+    transform types, in place, padded batch distance, planar, a scale factor, both precisions,
+    batches that do not fill the last tile."""
+    lib, be = gpu
+    K = B
+    st, text, _ = lib.describe(K.NOTINPLACE, K.REAL_FORWARD, K.DOUBLE, [4, 5], 1000)
+    assert st == 0 and "folded(3)" in text, text
+    for lengths, batch in (([4, 5], 1000), ([4, 5], 37), ([6, 10], 333), ([3, 3], 4097), ([5, 7, 3], 211), ([4, 5, 6], 100),
+                           ([12, 9], 65), ([2, 2, 2], 1001), ([20, 6], 50), ([33, 5], 77)):
+        for prec in (K.SINGLE, K.DOUBLE):
+            H.check(lib, be, K.COMPLEX_FORWARD, lengths, batch, prec)
+            H.check(lib, be, K.COMPLEX_INVERSE, lengths, batch, prec, inplace=True, scale=0.5)
+            H.check(lib, be, K.REAL_FORWARD, lengths, batch, prec)
+            H.check(lib, be, K.REAL_INVERSE, lengths, batch, prec)
+            H.check(lib, be, K.REAL_FORWARD, lengths, batch, prec, inplace=True)
+            H.check(lib, be, K.REAL_INVERSE, lengths, batch, prec, inplace=True)
+        total = int(np.prod(lengths))
+        strides = [1]
+        for v in lengths[:-1]:
+            strides.append(strides[-1] * v)
+        H.check(lib, be, K.COMPLEX_FORWARD, lengths, batch, K.SINGLE, in_strides=strides, in_dist=total + 3,
+                out_strides=strides, out_dist=total + 5)
+        H.check(lib, be, K.COMPLEX_FORWARD, lengths, batch, K.DOUBLE, in_type=K.COMPLEX_PLANAR,
+                out_type=K.COMPLEX_PLANAR)
+        H.check(lib, be, K.REAL_FORWARD, lengths, batch, K.SINGLE, out_type=K.HERMITIAN_PLANAR)
+
+
 def test_column_tiles_that_span_more_than_two_gib(gpu):
     """A column pass whose tile reaches from the first to the last byte of a 2 GiB array: element
     offsets inside the tile need 29 bits in single precision (129 x 2^21 elements), byte offsets 32."""

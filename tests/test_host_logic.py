@@ -227,6 +227,32 @@ def test_planar_arrays_take_the_compiled_kernels(emu):
     assert all(" lean" in p and " fast" in p and "planar" in p for p in ps), ps
 
 
+def test_short_rows_fold_the_batch_into_the_tile_axis(emu):
+    """A column pass over rows shorter than a tile takes (column, batch item) pairs as tile
+    entries; results through the run-time-schedule kernel of the emulated runtime."""
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4, 5], 1000)
+    assert st == 0 and "folded(4)" in text and "tile 64x5" in text, text
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4, 5, 6], 100)
+    assert st == 0 and "folded(4)" in text and "folded(20)" in text, text
+    # rows of 64 and more elements fill a tile by themselves
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [64, 5], 1000)
+    assert st == 0 and "folded" not in text, text
+    K = B
+    for lengths, batch in (([4, 5], 70), ([3, 3], 130), ([5, 7, 3], 9), ([6, 10], 21)):
+        H.check(emu, HOST, K.COMPLEX_FORWARD, lengths, batch, K.DOUBLE)
+        H.check(emu, HOST, K.COMPLEX_INVERSE, lengths, batch, K.SINGLE, inplace=True)
+        H.check(emu, HOST, K.REAL_FORWARD, lengths, batch, K.DOUBLE)
+        H.check(emu, HOST, K.REAL_INVERSE, lengths, batch, K.SINGLE, inplace=True)
+        total = int(np.prod(lengths))
+        strides = [1]
+        for v in lengths[:-1]:
+            strides.append(strides[-1] * v)
+        H.check(emu, HOST, K.COMPLEX_FORWARD, lengths, batch, K.SINGLE, in_strides=strides, in_dist=total + 3,
+                out_strides=strides, out_dist=total + 5)
+        H.check(emu, HOST, K.COMPLEX_FORWARD, lengths, batch, K.DOUBLE, in_type=K.COMPLEX_PLANAR,
+                out_type=K.COMPLEX_PLANAR)
+
+
 def test_pass_lists_of_the_benchmark_configurations(emu):
     st, text, work = emu.describe(B.INPLACE, B.COMPLEX_FORWARD, B.SINGLE, [4096], 1024)
     assert st == 0 and len(passes(text)) == 1 and work == 0 and "16x16x16" in text
