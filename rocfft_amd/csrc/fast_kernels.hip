@@ -22,7 +22,11 @@ namespace
 {
 
 // MODE 0: scalar accesses, every fused operation; 1: vector accesses, every fused operation;
-// 2: the lean path (vector accesses, interleaved complex on both sides)
+// 2: the lean path (vector accesses, complex arrays on both sides, every fused operation);
+// 3: the lean path for plain passes only (interleaved complex in and out, nothing fused but a
+// scale factor); 4: the same plus the large twiddle on the store side.  The variants 3 and 4 are
+// the lean kernel compiled under assumptions on its arguments (fast_assume_plain): the compiler
+// drops every other path, which leaves a fifth of the code and 10-50 registers fewer.
 // Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
 // their tile rows wide); no kernel here needs more than the 256 registers that leaves a thread.
 // The longest lengths need up to 1024 threads for one transform (128 registers a thread).
@@ -32,12 +36,38 @@ constexpr int fast_block_limit()
     return Cfg::TPT > 512 ? 1024 : 512;
 }
 
+// what fftrt_launch_fast_tile has checked on the host before it picks variant 3 or 4
+template <typename Cfg, int MODE>
+__device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
+{
+    if constexpr(MODE >= 3)
+    {
+        __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
+        __builtin_assume(p.store_op == FFTK_STORE_COMPLEX);
+        __builtin_assume(p.in_planar == 0);
+        __builtin_assume(p.out_planar == 0);
+        __builtin_assume(p.stage_io == 0);
+        __builtin_assume(p.w_inner == 0);
+        __builtin_assume(p.n_in == (uint32_t)Cfg::N);
+        __builtin_assume(p.n_out == (uint32_t)Cfg::N);
+        if constexpr(MODE == 3)
+        {
+            __builtin_assume((p.flags & ~(uint32_t)FFTK_F_SCALE) == 0);
+            __builtin_assume(p.aux_dim == 0);
+            __builtin_assume(p.oc0_first == 0);
+        }
+        else
+            __builtin_assume((p.flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0);
+    }
+}
+
 template <typename T, typename Cfg, int MODE>
 __global__ __launch_bounds__(fast_block_limit<Cfg>()) void fast_tile_kernel(const fftk_params p)
 {
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
-    fast_tile_body<T, Cfg, MODE != 0, MODE == 2>(p, reinterpret_cast<C*>(smem_raw));
+    fast_assume_plain<Cfg, MODE>(p);
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // The same kernel held to the registers that let WAVES waves share a SIMD.
@@ -46,11 +76,12 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
 {
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
-    fast_tile_body<T, Cfg, MODE != 0, MODE == 2>(p, reinterpret_cast<C*>(smem_raw));
+    fast_assume_plain<Cfg, MODE>(p);
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // Waves per SIMD a kernel is compiled for; 0 = whatever its natural register count gives.
-// Single precision, lean variant: four.  265 of these kernels take 129-160 registers by
+// Single precision, lean variants: four.  265 of the full lean kernels take 129-160 registers by
 // themselves, which leaves three waves a SIMD while their LDS tiles (about 33 KB) allow four
 // workgroups a compute unit; held to 128 registers (12-140 bytes of spill each) the transforms
 // that are bound by memory run 6 % faster on average and up to 24 %, none more than 5 % slower;
@@ -59,7 +90,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
 template <typename T, typename Cfg, int MODE>
 constexpr int fast_waves()
 {
-    return (sizeof(T) == 4 && MODE == 2 && Cfg::TPT <= 512) ? 4 : 0;
+    return (sizeof(T) == 4 && MODE >= 2 && Cfg::TPT <= 512) ? 4 : 0;
 }
 
 template <typename T, typename Cfg, int MODE>
@@ -83,10 +114,12 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* str
 // all_modes = 1: the three variants; 0: the lean one only
 #define FAST_ONE_1(T, P, N, A, B, C, D, TT)                                                            \
     {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 0>},
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 0>,        \
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>},
 #define FAST_ONE_0(T, P, N, A, B, C, D, TT)                                                            \
     {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
-     nullptr, nullptr},
+     nullptr, nullptr, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>,                                      \
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>},
 #define FAST_DBL_1(FULL, N, A, B, C, D, TTD) FAST_ONE_##FULL(double, 1, N, A, B, C, D, TTD)
 #define FAST_DBL_0(FULL, N, A, B, C, D, TTD)
 #define FAST_ENTRY(FULL, N, A, B, C, D, TTF, TTD, DBL) \
@@ -236,6 +269,15 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
     if(cnt != p->nf)
         return (int)hipErrorInvalidValue;
     fast_launch_fn fn = p->lean ? e->lean : vec ? e->vec : e->scalar;
+    if(p->lean && p->load_op == FFTK_LOAD_COMPLEX && p->store_op == FFTK_STORE_COMPLEX && !p->in_planar
+       && !p->out_planar && !p->stage_io && !p->w_inner && p->n_in == p->n && p->n_out == p->n)
+    {
+        // plain passes: the variants compiled for them alone (see fast_assume_plain)
+        if((p->flags & ~(uint32_t)FFTK_F_SCALE) == 0 && p->aux_dim == 0 && !p->oc0_first)
+            fn = e->plain;
+        else if((p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0)
+            fn = e->plain_tw;
+    }
     if(!fn)
         return FFTRT_NO_FAST_VARIANT;
     return fn(p, grid, lds_bytes, stream);
