@@ -24,9 +24,11 @@ namespace
 // MODE 0: scalar accesses, every fused operation; 1: vector accesses, every fused operation;
 // 2: the lean path (vector accesses, complex arrays on both sides, every fused operation);
 // 3: the lean path for plain passes only (interleaved complex in and out, nothing fused but a
-// scale factor); 4: the same plus the large twiddle on the store side.  The variants 3 and 4 are
-// the lean kernel compiled under assumptions on its arguments (fast_assume_plain): the compiler
-// drops every other path, which leaves a fifth of the code and 10-50 registers fewer.
+// scale factor); 4: the same plus the large twiddle on the store side; 5: plain passes, the
+// fused real pre/post-processing and the tile copy of short transforms, interleaved arrays.
+// The variants 3 to 5 are the lean kernel compiled under assumptions on its arguments
+// (fast_assume_plain): the compiler drops every other path, which leaves a fifth to a third of
+// the code and 10-50 registers fewer.
 // Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
 // their tile rows wide); no kernel here needs more than the 256 registers that leaves a thread.
 // The longest lengths need up to 1024 threads for one transform (128 registers a thread).
@@ -40,7 +42,18 @@ constexpr int fast_block_limit()
 template <typename Cfg, int MODE>
 __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
 {
-    if constexpr(MODE >= 3)
+    if constexpr(MODE == 5)
+    {
+        __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX || p.load_op == FFTK_LOAD_C2R_PRE);
+        __builtin_assume(p.store_op == FFTK_STORE_COMPLEX || p.store_op == FFTK_STORE_R2C_POST);
+        __builtin_assume((p.flags & ~(uint32_t)FFTK_F_SCALE) == 0);
+        __builtin_assume(p.in_planar == 0);
+        __builtin_assume(p.out_planar == 0);
+        __builtin_assume(p.w_inner == 0);
+        __builtin_assume(p.aux_dim == 0);
+        __builtin_assume(p.oc0_first == 0);
+    }
+    else if constexpr(MODE >= 3)
     {
         __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
         __builtin_assume(p.store_op == FFTK_STORE_COMPLEX);
@@ -115,11 +128,12 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* str
 #define FAST_ONE_1(T, P, N, A, B, C, D, TT)                                                            \
     {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
      &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 0>,        \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>},
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>,        \
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 5>},
 #define FAST_ONE_0(T, P, N, A, B, C, D, TT)                                                            \
     {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
      nullptr, nullptr, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>,                                      \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>},
+     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 5>},
 #define FAST_DBL_1(FULL, N, A, B, C, D, TTD) FAST_ONE_##FULL(double, 1, N, A, B, C, D, TTD)
 #define FAST_DBL_0(FULL, N, A, B, C, D, TTD)
 #define FAST_ENTRY(FULL, N, A, B, C, D, TTF, TTD, DBL) \
@@ -269,14 +283,19 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
     if(cnt != p->nf)
         return (int)hipErrorInvalidValue;
     fast_launch_fn fn = p->lean ? e->lean : vec ? e->vec : e->scalar;
-    if(p->lean && p->load_op == FFTK_LOAD_COMPLEX && p->store_op == FFTK_STORE_COMPLEX && !p->in_planar
-       && !p->out_planar && !p->stage_io && !p->w_inner && p->n_in == p->n && p->n_out == p->n)
+    // the variants compiled for some kinds of passes alone (see fast_assume_plain)
+    if(p->lean && !p->in_planar && !p->out_planar && !p->w_inner)
     {
-        // plain passes: the variants compiled for them alone (see fast_assume_plain)
-        if((p->flags & ~(uint32_t)FFTK_F_SCALE) == 0 && p->aux_dim == 0 && !p->oc0_first)
+        const bool plain_ops = p->load_op == FFTK_LOAD_COMPLEX && p->store_op == FFTK_STORE_COMPLEX && !p->stage_io
+                               && p->n_in == p->n && p->n_out == p->n;
+        const bool only_scale = (p->flags & ~(uint32_t)FFTK_F_SCALE) == 0 && p->aux_dim == 0 && !p->oc0_first;
+        if(plain_ops && only_scale)
             fn = e->plain;
-        else if((p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0)
+        else if(plain_ops && (p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0)
             fn = e->plain_tw;
+        else if(only_scale && (p->load_op == FFTK_LOAD_COMPLEX || p->load_op == FFTK_LOAD_C2R_PRE)
+                && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST))
+            fn = e->real;
     }
     if(!fn)
         return FFTRT_NO_FAST_VARIANT;

@@ -19,9 +19,9 @@ struct FastEntry
     // fused operation; scalar: scalar accesses.  A missing variant is null and the generic
     // kernel runs instead.
     fast_launch_fn lean, vec, scalar;
-    // the lean kernel compiled for plain passes only, and for plain passes with the large
-    // twiddle on the store side
-    fast_launch_fn plain, plain_tw;
+    // the lean kernel compiled for plain passes only, for plain passes with the large twiddle on
+    // the store side, and for passes with the fused real pre/post-processing or a tile copy
+    fast_launch_fn plain, plain_tw, real;
 };
 
 #endif
