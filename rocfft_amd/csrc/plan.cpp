@@ -713,8 +713,18 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     // A column pass over very short rows (a 4 x 5 transform: 4 columns) would leave most lanes of
     // its workgroups idle.  Fold the longest other plain axis (the transforms of a batch) into the
     // tile axis: tile entries are then (column, batch item) pairs.
-    if(g_fold_tiles && (k.in_fast_tile || k.out_fast_tile) && !tile_axis.aux && tile_axis.cnt < 64 && tile_axis.is >= 0
-       && tile_axis.os >= 0)
+    // (Only where the tiles would otherwise not fill one wave, or run less than 65 % full: a row
+    // count just below a power of two, or many threads per transform, keep the workgroups busy
+    // anyway, and folding measured 0-25 % slower there.)
+    bool fold_pays = false;
+    {
+        const uint32_t w_plain = std::min<uint32_t>(std::min<uint32_t>(64, floor_pow2(std::max<uint32_t>(1, 512 / sched_T))),
+                                                    ceil_pow2(tile_axis.cnt));
+        const uint64_t slots   = (uint64_t)((tile_axis.cnt + w_plain - 1) / w_plain) * w_plain;
+        fold_pays = (uint64_t)w_plain * sched_T < 64 || (double)tile_axis.cnt < 0.65 * (double)slots;
+    }
+    if(g_fold_tiles && (k.in_fast_tile || k.out_fast_tile) && !tile_axis.aux && fold_pays && tile_axis.cnt < 64
+       && tile_axis.is >= 0 && tile_axis.os >= 0)
     {
         int fold = -1;
         for(size_t i = 0; i < ax.size(); ++i)
