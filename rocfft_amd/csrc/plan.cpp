@@ -2473,7 +2473,17 @@ static rocfft_status build_exec_plan_once(const Problem& p, ExecPlan& plan, bool
                 uint64_t half = n0 / 2;
                 View     rv   = realpair_view(BUF_IN, p.istride, p.idist, p.ioffset, p.rank);
                 auto     oth  = other_axes(rv, hv, p.len, p.rank, p.batch, 0);
-                if(big_eligible(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io))
+                if(half == 1)
+                {
+                    // two real samples a row: no transform, the post-processing step alone
+                    // (bins x0 + x1 and x0 - x1) from the input to the output
+                    std::vector<Other> rows;
+                    for(const Other& o : oth)
+                        rows.push_back({o.cnt, o.is, o.os});
+                    emit_real_step(b, PASS_REAL_POST, half, rows, rv.stride[0], rv.io, hv.stride[0], hv.io, p.scale,
+                                   last0 && p.has_scale);
+                }
+                else if(big_eligible(b, half, rv.stride[0], hv.stride[0], oth, rv.io, hv.io))
                     emit_big(b, 1, oth, rv.io, hv.io, -1, p.scale, last0 && p.has_scale);
                 else if(single_kernel_length(half, b.esize)
                         && plain_dim_is_single(half, rv.stride[0] != 2, b.esize, rv.stride[0], hv.stride[0]))
@@ -2564,7 +2574,17 @@ static rocfft_status build_exec_plan_once(const Problem& p, ExecPlan& plan, bool
             uint64_t half = n0 / 2;
             View     rv   = realpair_view(out_buf, p.ostride, p.odist, p.ooffset, p.rank);
             auto     oth  = other_axes(hv, rv, p.len, p.rank, p.batch, 0);
-            if(big_eligible(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io))
+            if(half == 1)
+            {
+                // two real samples a row: the pre-processing step alone, from the input bins to the
+                // output
+                std::vector<Other> rows;
+                for(const Other& o : oth)
+                    rows.push_back({o.cnt, o.os, o.is});
+                emit_real_step(b, PASS_REAL_PRE, half, rows, rv.stride[0], rv.io, hv.stride[0], hv.io, p.scale,
+                               p.has_scale);
+            }
+            else if(big_eligible(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io))
                 emit_big(b, 2, oth, hv.io, rv.io, +1, p.scale, p.has_scale);
             else if(single_kernel_length(half, b.esize)
                     && (plan.inplace

@@ -679,10 +679,20 @@ FFT_DEV void real_pre_elem(const fftk_real_params& p, uint64_t gid)
         zq.x = u.x - v.x * t.y + u.y * t.x;
         zq.y = -v.y + u.y * t.y + v.x * t.x;
     }
+    if(p.use_scale)
+    {
+        zj.x *= (T)p.scale;
+        zj.y *= (T)p.scale;
+    }
     z0[zb + (int64_t)j * p.z_s] = zj.x;
     z1[zb + (int64_t)j * p.z_s] = zj.y;
     if(two)
     {
+        if(p.use_scale)
+        {
+            zq.x *= (T)p.scale;
+            zq.y *= (T)p.scale;
+        }
         z0[zb + (int64_t)jq * p.z_s] = zq.x;
         z1[zb + (int64_t)jq * p.z_s] = zq.y;
     }

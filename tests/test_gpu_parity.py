@@ -200,6 +200,21 @@ def test_short_rows_with_a_batch_fold_into_full_tiles(gpu):
         H.check(lib, be, K.REAL_FORWARD, lengths, batch, K.SINGLE, out_type=K.HERMITIAN_PLANAR)
 
 
+def test_real_rows_of_two_samples(gpu):
+    """Real transforms with two samples in the first dimension: the pre/post-processing pass alone
+    along that dimension, all layouts."""
+    lib, be = gpu
+    K = B
+    for lengths, batch in (([2], 1000), ([2, 64], 50), ([2, 91, 135], 3), ([2, 7], 4001)):
+        for prec in (K.SINGLE, K.DOUBLE):
+            H.check(lib, be, K.REAL_FORWARD, lengths, batch, prec)
+            H.check(lib, be, K.REAL_INVERSE, lengths, batch, prec)
+            H.check(lib, be, K.REAL_FORWARD, lengths, batch, prec, inplace=True, scale=0.5)
+            H.check(lib, be, K.REAL_INVERSE, lengths, batch, prec, inplace=True, scale=0.25)
+        H.check(lib, be, K.REAL_FORWARD, lengths, batch, K.DOUBLE, out_type=K.HERMITIAN_PLANAR)
+        H.check(lib, be, K.REAL_INVERSE, lengths, batch, K.SINGLE, in_type=K.HERMITIAN_PLANAR, scale=2.0)
+
+
 def test_column_tiles_that_span_more_than_two_gib(gpu):
     """A column pass whose tile reaches from the first to the last byte of a 2 GiB array: element
     offsets inside the tile need 29 bits in single precision (129 x 2^21 elements), byte offsets 32."""

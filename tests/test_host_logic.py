@@ -227,6 +227,22 @@ def test_planar_arrays_take_the_compiled_kernels(emu):
     assert all(" lean" in p and " fast" in p and "planar" in p for p in ps), ps
 
 
+def test_real_rows_of_two_samples(emu):
+    """Real transforms whose first dimension has two samples need no transform along it: one
+    pre/post-processing pass between the user's arrays."""
+    st, text, _ = emu.describe(B.NOTINPLACE, B.REAL_FORWARD, B.SINGLE, [2, 91, 135], 4)
+    assert st == 0 and len(passes(text)) == 3 and "n=1 " not in text, text
+    K = B
+    for lengths, batch in (([2], 5), ([2, 7], 3), ([2, 9, 5], 2)):
+        for prec in (K.SINGLE, K.DOUBLE):
+            H.check(emu, HOST, K.REAL_FORWARD, lengths, batch, prec)
+            H.check(emu, HOST, K.REAL_INVERSE, lengths, batch, prec)
+            H.check(emu, HOST, K.REAL_FORWARD, lengths, batch, prec, inplace=True, scale=0.5)
+            H.check(emu, HOST, K.REAL_INVERSE, lengths, batch, prec, inplace=True, scale=0.25)
+        H.check(emu, HOST, K.REAL_FORWARD, lengths, batch, K.DOUBLE, out_type=K.HERMITIAN_PLANAR)
+        H.check(emu, HOST, K.REAL_INVERSE, lengths, batch, K.SINGLE, in_type=K.HERMITIAN_PLANAR, scale=2.0)
+
+
 def test_short_rows_fold_the_batch_into_the_tile_axis(emu):
     """A column pass over rows shorter than a tile takes (column, batch item) pairs as tile
     entries; results through the run-time-schedule kernel of the emulated runtime."""
