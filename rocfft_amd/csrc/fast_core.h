@@ -435,7 +435,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     constexpr int                     PAIR_IT    = (PAIRS + Cfg::TPT - 1) / Cfg::TPT;
     constexpr bool                    PAIR_EXACT = PAIRS % Cfg::TPT == 0;
     // transforms whose lanes cover 16 contiguous bytes or less can go through LDS instead
-    constexpr bool                    STAGE_OK = Cfg::TPT == 1 || Cfg::TPT * sizeof(C) <= 16;
+    // (16 bytes of interleaved pairs, or of the scalars of a planar array)
+    constexpr bool                    STAGE_OK = Cfg::TPT == 1 || Cfg::TPT * sizeof(C) <= 32;
     constexpr int                     STAGE_IT = (N + Cfg::TPT - 1) / Cfg::TPT;
     constexpr int                     BINS_IT  = (N + 1 + Cfg::TPT - 1) / Cfg::TPT; // N+1 Hermitian bins per row
     // odd lengths also serve as odd-length real transforms (real samples on one side)
@@ -502,15 +503,19 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 staged               = true;
                 const uint32_t total = p.W * (uint32_t)(N + 1);
                 C              cp[BINS_IT];
-#pragma unroll
-                for(int i = 0; i < BINS_IT; ++i)
+                auto           copy_in = [&](auto in) __attribute__((always_inline))
                 {
-                    const uint32_t e     = tid + i * p.nthreads;
-                    const uint32_t w_    = e / (uint32_t)(N + 1);
-                    const uint32_t j_    = e - w_ * (uint32_t)(N + 1);
-                    const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
-                    cp[i]                = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
-                }
+#pragma unroll
+                    for(int i = 0; i < BINS_IT; ++i)
+                    {
+                        const uint32_t e     = tid + i * p.nthreads;
+                        const uint32_t w_    = e / (uint32_t)(N + 1);
+                        const uint32_t j_    = e - w_ * (uint32_t)(N + 1);
+                        const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
+                        cp[i]                = in.at(valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u);
+                    }
+                };
+                FK_WITH_IN(copy_in);
                 // unconditional stores (a condition would pull each load next to its store and make
                 // the thread wait for one load after the other): the LDS allocation of such a pass
                 // covers BINS_IT * nthreads elements
@@ -649,16 +654,20 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         // consecutive lanes copy consecutive elements of the tile into LDS
         const uint32_t total = p.W * N;
         // every load is issued before the first value is used
-        C cp[STAGE_IT];
-#pragma unroll
-        for(int i = 0; i < STAGE_IT; ++i)
+        C    cp[STAGE_IT];
+        auto copy_in = [&](auto in) __attribute__((always_inline))
         {
-            const uint32_t e     = tid + i * p.nthreads;
-            const uint32_t w_    = e / (uint32_t)N;
-            const uint32_t j_    = e - w_ * (uint32_t)N;
-            const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
-            cp[i]                = src[valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u];
-        }
+#pragma unroll
+            for(int i = 0; i < STAGE_IT; ++i)
+            {
+                const uint32_t e     = tid + i * p.nthreads;
+                const uint32_t w_    = e / (uint32_t)N;
+                const uint32_t j_    = e - w_ * (uint32_t)N;
+                const bool     valid = e < total && c.tile0 + w_ < p.tile_cnt;
+                cp[i]                = in.at(valid ? j_ * p.t_is_c + w_ * p.w_is_c : 0u);
+            }
+        };
+        FK_WITH_IN(copy_in);
         // unconditional stores, as above: the LDS allocation covers the rows up to
         // (STAGE_IT * nthreads - 1) / N
 #pragma unroll
@@ -912,15 +921,19 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 }
                 __syncthreads();
                 const uint32_t total = p.W * (uint32_t)(N + 1);
-#pragma unroll
-                for(int i = 0; i < BINS_IT; ++i)
+                auto copy_out = [&](auto out) __attribute__((always_inline))
                 {
-                    const uint32_t e  = tid + i * p.nthreads;
-                    const uint32_t w_ = e / (uint32_t)(N + 1);
-                    const uint32_t j_ = e - w_ * (uint32_t)(N + 1);
-                    if(e < total && c.tile0 + w_ < p.tile_cnt)
-                        dst[j_ * p.t_os_c + w_ * p.w_os_c] = lds[e];
-                }
+#pragma unroll
+                    for(int i = 0; i < BINS_IT; ++i)
+                    {
+                        const uint32_t e  = tid + i * p.nthreads;
+                        const uint32_t w_ = e / (uint32_t)(N + 1);
+                        const uint32_t j_ = e - w_ * (uint32_t)(N + 1);
+                        if(e < total && c.tile0 + w_ < p.tile_cnt)
+                            out.put(j_ * p.t_os_c + w_ * p.w_os_c, lds[e]);
+                    }
+                };
+                FK_WITH_OUT(copy_out);
                 return;
             }
         }
@@ -1012,7 +1025,10 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     v = c_swap(v);
                 v.x *= sc;
                 v.y *= sc;
-                dst[j_ * p.t_os_c + w_ * p.w_os_c] = v;
+                if(p.out_planar)
+                    out_planar.put(j_ * p.t_os_c + w_ * p.w_os_c, v);
+                else
+                    dst[j_ * p.t_os_c + w_ * p.w_os_c] = v;
             }
         }
         return;

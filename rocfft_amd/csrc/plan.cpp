@@ -956,8 +956,10 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
                 const bool plain_ops = s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_COMPLEX;
                 const bool real_ops  = (s.load_op == FFTK_LOAD_COMPLEX && s.store_op == FFTK_STORE_R2C_POST)
                                       || (s.load_op == FFTK_LOAD_C2R_PRE && s.store_op == FFTK_STORE_COMPLEX);
-                if(!column && (k.T == 1 || ((size_t)k.T * esize <= 16 && k.n < 32)) && k.t_is == 2 && k.t_os == 2
-                   && in_kind == 1 && out_kind == 1
+                // (lanes of a transform that together cover 16 bytes or less per access)
+                const size_t access = (in_kind == 2 || out_kind == 2) ? esize / 2 : esize;
+                if(!column && (k.T == 1 || ((size_t)k.T * access <= 16 && k.n < 32)) && k.t_is == (in_kind == 1 ? 2 : 1)
+                   && k.t_os == (out_kind == 1 ? 2 : 1) && in_kind <= 2 && out_kind <= 2
                    && (plain_ops || real_ops) && (k.flags & ~(uint32_t)FFTK_F_SCALE) == 0 && k.n_in == k.n
                    && k.n_out == k.n)
                 {
