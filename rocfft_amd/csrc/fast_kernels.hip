@@ -124,62 +124,49 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* str
     return (int)hipGetLastError();
 }
 
-// all_modes = 1: the three variants; 0: the lean one only
-#define FAST_ONE_1(T, P, N, A, B, C, D, TT)                                                            \
-    {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 1>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 0>,        \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>,        \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 5>},
-#define FAST_ONE_0(T, P, N, A, B, C, D, TT)                                                            \
-    {P, N, {A, B, C, D}, FastCfg<N, A, B, C, D, TT>::TPT, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 2>,  \
-     nullptr, nullptr, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 3>,                                      \
-     &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 4>, &launch_fast<T, FastCfg<N, A, B, C, D, TT>, 5>},
-#define FAST_DBL_1(FULL, N, A, B, C, D, TTD) FAST_ONE_##FULL(double, 1, N, A, B, C, D, TTD)
-#define FAST_DBL_0(FULL, N, A, B, C, D, TTD)
-#define FAST_ENTRY(FULL, N, A, B, C, D, TTF, TTD, DBL) \
-    FAST_ONE_##FULL(float, 0, N, A, B, C, D, TTF) FAST_DBL_##DBL(FULL, N, A, B, C, D, TTD)
+// The variants 4 and 5 exist only in single precision, where the registers they save lift the
+// number of waves, and up to 4096 points: the longer kernels seldom run such passes, and every
+// variant costs build time.  The variants 0 and 1 exist for the lengths marked all_modes.
+template <typename T, typename Cfg, int MODE, bool WANTED>
+constexpr fast_launch_fn fast_variant()
+{
+    if constexpr(WANTED)
+        return &launch_fast<T, Cfg, MODE>;
+    else
+        return nullptr;
+}
 
-#define FAST_PICK_0(...)
-#define FAST_PICK_1(...)
-#define FAST_PICK_2(...)
-#define FAST_PICK_3(...)
-#define FAST_PICK_4(...)
-#define FAST_PICK_5(...)
-#define FAST_PICK_6(...)
-#define FAST_PICK_7(...)
-#if FAST_SLICE == 0
-#undef FAST_PICK_0
-#define FAST_PICK_0(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 1
-#undef FAST_PICK_1
-#define FAST_PICK_1(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 2
-#undef FAST_PICK_2
-#define FAST_PICK_2(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 3
-#undef FAST_PICK_3
-#define FAST_PICK_3(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 4
-#undef FAST_PICK_4
-#define FAST_PICK_4(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 5
-#undef FAST_PICK_5
-#define FAST_PICK_5(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 6
-#undef FAST_PICK_6
-#define FAST_PICK_6(...) FAST_ENTRY(__VA_ARGS__)
-#elif FAST_SLICE == 7
-#undef FAST_PICK_7
-#define FAST_PICK_7(...) FAST_ENTRY(__VA_ARGS__)
-#else
-#error "FAST_SLICE out of range"
-#endif
-#define FAST_SCHED(SLICE, ...) FAST_PICK_##SLICE(__VA_ARGS__)
+// the table entry of one kernel family, or an empty entry (n = 0) in the translation units
+// that do not instantiate it
+template <int SLICE, typename T, int PRECISION, int ALL_MODES, bool EXISTS, typename Cfg>
+constexpr FastEntry fast_entry()
+{
+    if constexpr(SLICE == FAST_SLICE && EXISTS)
+    {
+        constexpr bool more = Cfg::N <= 4096 && sizeof(T) == 4;
+        return FastEntry{PRECISION,
+                         (uint32_t)Cfg::N,
+                         {(uint32_t)Cfg::R0, (uint32_t)Cfg::R1, (uint32_t)Cfg::R2, (uint32_t)Cfg::R3},
+                         (uint32_t)Cfg::TPT,
+                         &launch_fast<T, Cfg, 2>,
+                         fast_variant<T, Cfg, 1, ALL_MODES != 0>(),
+                         fast_variant<T, Cfg, 0, ALL_MODES != 0>(),
+                         &launch_fast<T, Cfg, 3>,
+                         fast_variant<T, Cfg, 4, more>(),
+                         fast_variant<T, Cfg, 5, more>()};
+    }
+    else
+        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+}
+
+#define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD, DBL)                  \
+    fast_entry<SLICE, float, 0, FULL, true, FastCfg<N, A, B, C, D, TTF>>(),     \
+        fast_entry<SLICE, double, 1, FULL, (DBL) != 0, FastCfg<N, A, B, C, D, (DBL) ? TTD : TTF>>(),
 
 const FastEntry g_slice[] = {
 #include "fast_schedules.h"
 };
-static_assert(FAST_SLICES == 8, "the FAST_PICK_ list above covers eight slices");
+static_assert(FAST_SLICE >= 0 && FAST_SLICE < FAST_SLICES, "compile with -DFAST_SLICE=0..FAST_SLICES-1");
 
 } // namespace
 
@@ -193,13 +180,10 @@ extern "C" const FastEntry* FAST_SLICE_FN(FAST_SLICE)(int* count)
 }
 
 #if FAST_SLICE == 0
-extern "C" const FastEntry* fftrt_fast_slice_1(int*);
-extern "C" const FastEntry* fftrt_fast_slice_2(int*);
-extern "C" const FastEntry* fftrt_fast_slice_3(int*);
-extern "C" const FastEntry* fftrt_fast_slice_4(int*);
-extern "C" const FastEntry* fftrt_fast_slice_5(int*);
-extern "C" const FastEntry* fftrt_fast_slice_6(int*);
-extern "C" const FastEntry* fftrt_fast_slice_7(int*);
+#define FAST_SLICE_LIST(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15)
+static_assert(FAST_SLICES == 16, "FAST_SLICE_LIST names sixteen slices");
+#define FAST_DECLARE(I) extern "C" const FastEntry* fftrt_fast_slice_##I(int*);
+FAST_SLICE_LIST(FAST_DECLARE)
 
 namespace
 {
@@ -213,15 +197,15 @@ const std::vector<const FastEntry*>& fast_index()
     static std::once_flag                once;
     std::call_once(once, []() {
         typedef const FastEntry* (*slice_fn)(int*);
-        const slice_fn slices[FAST_SLICES]
-            = {fftrt_fast_slice_0, fftrt_fast_slice_1, fftrt_fast_slice_2, fftrt_fast_slice_3,
-               fftrt_fast_slice_4, fftrt_fast_slice_5, fftrt_fast_slice_6, fftrt_fast_slice_7};
+#define FAST_NAME(I) fftrt_fast_slice_##I,
+        const slice_fn slices[FAST_SLICES] = {FAST_SLICE_LIST(FAST_NAME)};
         for(slice_fn f : slices)
         {
             int              cnt = 0;
             const FastEntry* e   = f(&cnt);
             for(int i = 0; i < cnt; ++i)
-                index.push_back(e + i);
+                if(e[i].n != 0) // (empty: instantiated in another slice, or no such kernel)
+                    index.push_back(e + i);
         }
         std::stable_sort(index.begin(), index.end(), [](const FastEntry* a, const FastEntry* b) {
             return a->precision != b->precision ? a->precision < b->precision : a->n < b->n;
@@ -291,10 +275,10 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
         const bool only_scale = (p->flags & ~(uint32_t)FFTK_F_SCALE) == 0 && p->aux_dim == 0 && !p->oc0_first;
         if(plain_ops && only_scale)
             fn = e->plain;
-        else if(plain_ops && (p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0)
+        else if(plain_ops && (p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0 && e->plain_tw)
             fn = e->plain_tw;
         else if(only_scale && (p->load_op == FFTK_LOAD_COMPLEX || p->load_op == FFTK_LOAD_C2R_PRE)
-                && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST))
+                && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST) && e->real)
             fn = e->real;
     }
     if(!fn)
