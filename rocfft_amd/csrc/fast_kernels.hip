@@ -94,16 +94,16 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
 }
 
 // Waves per SIMD a kernel is compiled for; 0 = whatever its natural register count gives.
-// Single precision, lean variants: four.  265 of the full lean kernels take 129-160 registers by
-// themselves, which leaves three waves a SIMD while their LDS tiles (about 33 KB) allow four
-// workgroups a compute unit; held to 128 registers (12-140 bytes of spill each) the transforms
-// that are bound by memory run 6 % faster on average and up to 24 %, none more than 5 % slower;
-// kernels below 128 registers are not affected.  (The 4096-point kernel: 138 registers; a batch
-// of 1024 on 256 compute units needs four workgroups a unit to run in one round.)
+// The single-precision variants 3 to 5 are built for four waves (128 registers): their LDS tiles
+// (about 33 KB) allow four workgroups a compute unit, and most of them fit without spilling (the
+// 4096-point plain kernel: 126 registers; a batch of 1024 on 256 compute units needs four
+// workgroups a unit to run in one round).  The full lean kernel keeps its natural count (129-160
+// registers for 265 lengths): held to 128 it spills 12-140 bytes a lane, and the passes that
+// still run on it (chirp-z, planar, odd-length real, folded tiles) measured the same either way.
 template <typename T, typename Cfg, int MODE>
 constexpr int fast_waves()
 {
-    return (sizeof(T) == 4 && MODE >= 2 && Cfg::TPT <= 512) ? 4 : 0;
+    return (sizeof(T) == 4 && MODE >= 3 && Cfg::TPT <= 512) ? 4 : 0;
 }
 
 template <typename T, typename Cfg, int MODE>
