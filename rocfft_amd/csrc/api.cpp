@@ -456,6 +456,9 @@ rocfft_status rocfft_plan_create(rocfft_plan* plan, rocfft_result_placement plac
 
 // static_work: take the work area from the library's device-resident array instead of the
 // caller's buffer or a fresh allocation, and refuse whatever would need an allocation
+// ROCFFT_AMD_NO_HALF_FUSE=1: half-precision arrays are always converted in separate passes
+static const bool g_no_half_fuse = getenv("ROCFFT_AMD_NO_HALF_FUSE") != nullptr;
+
 static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], void* out_buffer[],
                                   rocfft_execution_info info, float* pass_ms, bool static_work = false)
 {
@@ -572,6 +575,7 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         const bool out_complex = pr.out_type != rocfft_array_type_real && !out_planar;
         const int  nin = in_planar ? 2 : 1, nout = out_planar ? 2 : 1;
         bool       stage_in = false, stage_out = false;
+        ExecHalf   ehalf;
         if(staging)
         {
             if(have_cb && (in_planar || out_planar || half_io))
@@ -650,8 +654,22 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
                 if(want_work)
                     work = set.work;
             }
+            // half precision: a first (last) pass that converts on load (store) takes the user's
+            // array itself, and the copy on that side is not made
+            if(half_io && !g_no_half_fuse)
+            {
+                void* s_in[2]  = {st_in[0], st_in[1]};
+                void* s_out[2] = {st_out[0], st_out[1]};
+                if(&select_exec_plan(ep, s_in, s_out, work) == &ep)
+                {
+                    ehalf.in       = in[0];
+                    ehalf.out      = out[0];
+                    ehalf.fuse_in  = !in_planar && half_fusable(ep, true, in[0]);
+                    ehalf.fuse_out = !out_planar && half_fusable(ep, false, out[0]);
+                }
+            }
             bool ok = true;
-            for(int i = 0; i < nin && ok && stage_in; ++i)
+            for(int i = 0; i < nin && ok && stage_in && !ehalf.fuse_in; ++i)
             {
                 cin.store   = 0;
                 cin.offset  = (int64_t)pr.ioffset[i];
@@ -668,8 +686,9 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         }
         void* run_in[2]  = {stage_in ? st_in[0] : in[0], stage_in ? st_in[1] : in[1]};
         void* run_out[2] = {stage_out ? st_out[0] : out[0], stage_out ? st_out[1] : out[1]};
-        rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms, fused ? &ecb : nullptr);
-        for(int i = 0; i < nout && st == rocfft_status_success && stage_out; ++i)
+        rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms, fused ? &ecb : nullptr,
+                                         (ehalf.fuse_in || ehalf.fuse_out) ? &ehalf : nullptr);
+        for(int i = 0; i < nout && st == rocfft_status_success && stage_out && !ehalf.fuse_out; ++i)
         {
             cout.store   = 1;
             cout.offset  = (int64_t)pr.ooffset[i];

@@ -378,6 +378,59 @@ struct FkPlanarOut
     }
 };
 
+// interleaved pairs of IEEE half values (the arrays of a half-precision plan, which computes in
+// single precision): converted on the way in and rounded on the way out
+template <typename T>
+struct FkHalfIn
+{
+    typedef typename cplx_of<T>::type C;
+    const fft_half2* p;
+    const fft_half2* first;
+    static FFT_DEV C widen(fft_half2 h)
+    {
+        C v;
+        v.x = (T)h.x;
+        v.y = (T)h.y;
+        return v;
+    }
+    FFT_DEV C at(uint32_t off) const
+    {
+        return widen(p[off]);
+    }
+    FFT_DEV C at2(uint64_t a, uint32_t b) const
+    {
+        const fft_half2* pk = p + a;
+        return widen(pk[b]);
+    }
+    FFT_DEV C at_or_first(bool valid, uint32_t off) const
+    {
+        const fft_half2* pj = valid ? p + off : first;
+        return widen(*pj);
+    }
+};
+template <typename T>
+struct FkHalfOut
+{
+    typedef typename cplx_of<T>::type C;
+    fft_half2* p;
+    static FFT_DEV fft_half2 narrow(C v)
+    {
+        fft_half2 h;
+        h.x = (_Float16)v.x;
+        h.y = (_Float16)v.y;
+        return h;
+    }
+    FFT_DEV void put(uint32_t off, C v) const
+    {
+        p[off] = narrow(v);
+    }
+    FFT_DEV void put2(uint64_t a, uint32_t b, C v) const
+    {
+        fft_half2* pk = p + a;
+        pk[b]         = narrow(v);
+    }
+};
+
 // only the real part is written (offsets count scalars)
 template <typename T>
 struct FkRealOut
@@ -417,7 +470,7 @@ FFT_DEV uint32_t fk_w_out(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
 // Bluestein chirp on either side, convolution mode, the fused real pre/post-processing,
 // row-in/column-out passes and (odd lengths) real samples on one side with the half spectrum
 // on the other.
-template <typename T, typename Cfg>
+template <typename T, typename Cfg, bool HALF = false>
 __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cplx_of<T>::type* lds,
                                                const TileCtx<T>& c, uint32_t tid, uint32_t w,
                                                uint32_t tt, bool active)
@@ -452,23 +505,37 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     const FkPlanarIn<T>  in_planar{static_cast<const T*>(p.in0) + c.ibase, static_cast<const T*>(p.in1) + c.ibase,
                                   static_cast<const T*>(p.in0), static_cast<const T*>(p.in1)};
     const FkPairsOut<T>  out_pairs{dst};
+    // (HALF: in0 / out0 may point at half values; ibase / obase count scalars of that array)
+    const FkHalfIn<T>    in_half{reinterpret_cast<const fft_half2*>(static_cast<const _Float16*>(p.in0) + c.ibase),
+                              static_cast<const fft_half2*>(p.in0)};
+    const FkHalfOut<T>   out_half{reinterpret_cast<fft_half2*>(static_cast<_Float16*>(p.out0) + c.obase)};
     const FkPlanarOut<T> out_planar{static_cast<T*>(p.out0) + c.obase, static_cast<T*>(p.out1) + c.obase};
 // runs body(accessor) with the accessor of the side's array kind
-#define FK_WITH_IN(body)     \
-    do                       \
-    {                        \
-        if(p.in_planar)      \
-            body(in_planar); \
-        else                 \
-            body(in_pairs);  \
+#define FK_WITH_IN(body)            \
+    do                              \
+    {                               \
+        if(HALF && p.in_half)       \
+        {                           \
+            if constexpr(HALF)      \
+                body(in_half);      \
+        }                           \
+        else if(p.in_planar)        \
+            body(in_planar);        \
+        else                        \
+            body(in_pairs);         \
     } while(0)
-#define FK_WITH_OUT(body)     \
-    do                        \
-    {                         \
-        if(p.out_planar)      \
-            body(out_planar); \
-        else                  \
-            body(out_pairs);  \
+#define FK_WITH_OUT(body)           \
+    do                              \
+    {                               \
+        if(HALF && p.out_half)      \
+        {                           \
+            if constexpr(HALF)      \
+                body(out_half);     \
+        }                           \
+        else if(p.out_planar)       \
+            body(out_planar);       \
+        else                        \
+            body(out_pairs);        \
     } while(0)
 
     // ---------------------------------------------------------------- load
@@ -1025,10 +1092,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     v = c_swap(v);
                 v.x *= sc;
                 v.y *= sc;
-                if(p.out_planar)
-                    out_planar.put(j_ * p.t_os_c + w_ * p.w_os_c, v);
-                else
-                    dst[j_ * p.t_os_c + w_ * p.w_os_c] = v;
+                auto put = [&](auto out) __attribute__((always_inline)) { out.put(j_ * p.t_os_c + w_ * p.w_os_c, v); };
+                FK_WITH_OUT(put);
             }
         }
         return;
@@ -1165,7 +1230,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
 #undef FK_WITH_OUT
 }
 
-template <typename T, typename Cfg, bool VEC, bool LEAN>
+template <typename T, typename Cfg, bool VEC, bool LEAN, bool HALF = false>
 __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cplx_of<T>::type* lds)
 {
     typedef typename cplx_of<T>::type C;
@@ -1191,7 +1256,7 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
     }
     if constexpr(LEAN)
     {
-        fast_tile_lean<T, Cfg>(p, lds, c, tid, w, tt, active);
+        fast_tile_lean<T, Cfg, HALF>(p, lds, c, tid, w, tt, active);
         return;
     }
     C    r[Cfg::EPT];

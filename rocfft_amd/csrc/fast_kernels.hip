@@ -24,11 +24,12 @@ namespace
 // MODE 0: scalar accesses, every fused operation; 1: vector accesses, every fused operation;
 // 2: the lean path (vector accesses, complex arrays on both sides, every fused operation);
 // 3: the lean path for plain passes only (interleaved complex in and out, nothing fused but a
-// scale factor); 4: the same plus the large twiddle on the store side; 5: plain passes, the
-// fused real pre/post-processing and the tile copy of short transforms, interleaved arrays.
-// The variants 3 to 5 are the lean kernel compiled under assumptions on its arguments
-// (fast_assume_plain): the compiler drops every other path, which leaves a fifth to a third of
-// the code and 10-50 registers fewer.
+// scale factor); 4: interleaved arrays, a scale factor, the large twiddle on the store side, the
+// fused real pre/post-processing, the tile copy of short transforms, and (single precision)
+// arrays of IEEE half pairs on the load or the store side: the first and last pass of a
+// half-precision plan, which computes in single precision.  The variants 3 and 4 are the lean
+// kernel compiled under assumptions on its arguments (fast_assume_plain): the compiler drops
+// every other path, which leaves a fifth to a third of the code and 10-50 registers fewer.
 // Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
 // their tile rows wide); no kernel here needs more than the 256 registers that leaves a thread.
 // The longest lengths need up to 1024 threads for one transform (128 registers a thread).
@@ -42,18 +43,16 @@ constexpr int fast_block_limit()
 template <typename Cfg, int MODE>
 __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
 {
-    if constexpr(MODE == 5)
+    if constexpr(MODE == 4)
     {
         __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX || p.load_op == FFTK_LOAD_C2R_PRE);
         __builtin_assume(p.store_op == FFTK_STORE_COMPLEX || p.store_op == FFTK_STORE_R2C_POST);
-        __builtin_assume((p.flags & ~(uint32_t)FFTK_F_SCALE) == 0);
+        __builtin_assume((p.flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0);
         __builtin_assume(p.in_planar == 0);
         __builtin_assume(p.out_planar == 0);
         __builtin_assume(p.w_inner == 0);
-        __builtin_assume(p.aux_dim == 0);
-        __builtin_assume(p.oc0_first == 0);
     }
-    else if constexpr(MODE >= 3)
+    else if constexpr(MODE == 3)
     {
         __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
         __builtin_assume(p.store_op == FFTK_STORE_COMPLEX);
@@ -63,14 +62,9 @@ __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
         __builtin_assume(p.w_inner == 0);
         __builtin_assume(p.n_in == (uint32_t)Cfg::N);
         __builtin_assume(p.n_out == (uint32_t)Cfg::N);
-        if constexpr(MODE == 3)
-        {
-            __builtin_assume((p.flags & ~(uint32_t)FFTK_F_SCALE) == 0);
-            __builtin_assume(p.aux_dim == 0);
-            __builtin_assume(p.oc0_first == 0);
-        }
-        else
-            __builtin_assume((p.flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0);
+        __builtin_assume((p.flags & ~(uint32_t)FFTK_F_SCALE) == 0);
+        __builtin_assume(p.aux_dim == 0);
+        __builtin_assume(p.oc0_first == 0);
     }
 }
 
@@ -80,7 +74,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>()) void fast_tile_kernel(cons
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
     fast_assume_plain<Cfg, MODE>(p);
-    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // The same kernel held to the registers that let WAVES waves share a SIMD.
@@ -90,7 +84,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
     fast_assume_plain<Cfg, MODE>(p);
-    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // Waves per SIMD a kernel is compiled for; 0 = whatever its natural register count gives.
@@ -124,9 +118,10 @@ int launch_fast(const fftk_params* p, uint32_t grid, size_t lds_bytes, void* str
     return (int)hipGetLastError();
 }
 
-// The variants 4 and 5 exist only in single precision, where the registers they save lift the
-// number of waves, and up to 4096 points: the longer kernels seldom run such passes, and every
-// variant costs build time.  The variants 0 and 1 exist for the lengths marked all_modes.
+// Variant 4 exists in single precision up to 4096 points (where the registers it saves lift the
+// number of waves, and where half-precision arrays are taken in place: the longer kernels
+// seldom run such passes, and every variant costs build time).  The variants 0 and 1 exist for
+// the lengths marked all_modes.
 template <typename T, typename Cfg, int MODE, bool WANTED>
 constexpr fast_launch_fn fast_variant()
 {
@@ -152,11 +147,10 @@ constexpr FastEntry fast_entry()
                          fast_variant<T, Cfg, 1, ALL_MODES != 0>(),
                          fast_variant<T, Cfg, 0, ALL_MODES != 0>(),
                          &launch_fast<T, Cfg, 3>,
-                         fast_variant<T, Cfg, 4, more>(),
-                         fast_variant<T, Cfg, 5, more>()};
+                         fast_variant<T, Cfg, 4, more>()};
     }
     else
-        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr};
 }
 
 #define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD, DBL)                  \
@@ -180,8 +174,10 @@ extern "C" const FastEntry* FAST_SLICE_FN(FAST_SLICE)(int* count)
 }
 
 #if FAST_SLICE == 0
-#define FAST_SLICE_LIST(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15)
-static_assert(FAST_SLICES == 16, "FAST_SLICE_LIST names sixteen slices");
+#define FAST_SLICE_LIST(X)                                                                              \
+    X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16) X(17) X(18) \
+        X(19) X(20) X(21) X(22) X(23)
+static_assert(FAST_SLICES == 24, "FAST_SLICE_LIST names twenty-four slices");
 #define FAST_DECLARE(I) extern "C" const FastEntry* fftrt_fast_slice_##I(int*);
 FAST_SLICE_LIST(FAST_DECLARE)
 
@@ -252,6 +248,13 @@ extern "C" uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* rad
     return e->tpt;
 }
 
+// is there a compiled kernel of this length that reads or writes half-precision arrays?
+extern "C" int fftrt_fast_takes_half(uint32_t n)
+{
+    const FastEntry* e = find_fast(0, n);
+    return e && e->more ? 1 : 0;
+}
+
 // called by fftrt_launch_tile (kernels.hip) when the plan asked for the fast kernel;
 // returns FFTRT_NO_FAST_VARIANT when this access mode has no compiled variant
 extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
@@ -267,6 +270,13 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
     if(cnt != p->nf)
         return (int)hipErrorInvalidValue;
     fast_launch_fn fn = p->lean ? e->lean : vec ? e->vec : e->scalar;
+    if(p->in_half || p->out_half)
+    {
+        // (the planner offers such passes only after fftrt_fast_takes_half said yes)
+        if(!p->lean || !e->more)
+            return (int)hipErrorInvalidValue;
+        return e->more(p, grid, lds_bytes, stream);
+    }
     // the variants compiled for some kinds of passes alone (see fast_assume_plain);
     // ROCFFT_AMD_NO_VARIANTS=1 keeps every pass on the full lean kernel (for comparisons)
     static const bool variants = !getenv("ROCFFT_AMD_NO_VARIANTS");
@@ -277,11 +287,10 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
         const bool only_scale = (p->flags & ~(uint32_t)FFTK_F_SCALE) == 0 && p->aux_dim == 0 && !p->oc0_first;
         if(plain_ops && only_scale)
             fn = e->plain;
-        else if(plain_ops && (p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0 && e->plain_tw)
-            fn = e->plain_tw;
-        else if(only_scale && (p->load_op == FFTK_LOAD_COMPLEX || p->load_op == FFTK_LOAD_C2R_PRE)
-                && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST) && e->real)
-            fn = e->real;
+        else if(e->more && (p->flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0
+                && (p->load_op == FFTK_LOAD_COMPLEX || p->load_op == FFTK_LOAD_C2R_PRE)
+                && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST))
+            fn = e->more;
     }
     if(!fn)
         return FFTRT_NO_FAST_VARIANT;

@@ -19,9 +19,10 @@ struct FastEntry
     // fused operation; scalar: scalar accesses.  A missing variant is null and the generic
     // kernel runs instead.
     fast_launch_fn lean, vec, scalar;
-    // the lean kernel compiled for plain passes only, for plain passes with the large twiddle on
-    // the store side, and for passes with the fused real pre/post-processing or a tile copy
-    fast_launch_fn plain, plain_tw, real;
+    // the lean kernel compiled for plain passes only, and for the other passes over interleaved
+    // arrays without a chirp (twiddle on the store side, real pre/post-processing, tile copies,
+    // half-precision arrays on the user's side)
+    fast_launch_fn plain, more;
 };
 
 #endif

@@ -33,6 +33,9 @@ int fftrt_stream_capturing(void* stream);
 // then).  The threads per transform follow the generic kernel's rule, so a pass planned
 // for a fast kernel can run on the generic one when an access mode has no fast variant.
 uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* radix, uint32_t* nf);
+// 1 when a compiled single-precision kernel of length n can read or write arrays of IEEE half
+// pairs (the user's arrays of a half-precision plan)
+int fftrt_fast_takes_half(uint32_t n);
 // returned by the fast launcher when the requested access mode has no compiled variant
 #define FFTRT_NO_FAST_VARIANT (-2)
 

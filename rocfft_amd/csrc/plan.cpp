@@ -2786,13 +2786,54 @@ bool callbacks_fusable(const ExecPlan& plan, void* const in[2], void* const out[
     return true;
 }
 
+// the passes whose user side may be an array of half pairs: what variant 6 of the compiled
+// kernels covers (fast_kernels.hip)
+static bool pass_takes_half(const PassRec& r)
+{
+    if(r.kind != PASS_TILE || !r.kp.fast || !r.lean_ok)
+        return false;
+    const fftk_params& k = r.kp;
+    return (k.load_op == FFTK_LOAD_COMPLEX || k.load_op == FFTK_LOAD_C2R_PRE)
+           && (k.store_op == FFTK_STORE_COMPLEX || k.store_op == FFTK_STORE_R2C_POST)
+           && (k.flags & ~(uint32_t)(FFTK_F_SCALE | FFTK_F_TWIDDLE_STORE)) == 0 && !k.in_planar && !k.out_planar
+           && !k.w_inner && k.n_in == k.n && k.n_out == k.n && fftrt_fast_takes_half(k.n) != 0;
+}
+
+bool half_fusable(const ExecPlan& plan, bool input, const void* user)
+{
+    if(plan.precision != 0 || plan.passes.empty() || !user)
+        return false;
+    const PassRec& r  = input ? plan.passes.front() : plan.passes.back();
+    const IoRef&   io = input ? r.src : r.dst;
+    const int      want = input || plan.inplace ? BUF_IN : BUF_OUT;
+    if(!pass_takes_half(r) || io.buf != want || io.planar || io.im_delta != 1)
+        return false;
+    if(input)
+    {
+        // every later pass that reads the input array must find it rewritten (in single
+        // precision, in the scratch copy) by an earlier one
+        bool rewritten = false;
+        for(size_t i = 0; i < plan.passes.size(); ++i)
+        {
+            if(i > 0 && plan.passes[i].src.buf == BUF_IN && !rewritten)
+                return false;
+            if(plan.passes[i].dst.buf == BUF_IN)
+                rewritten = true;
+        }
+    }
+    // a pair of half values is one 4-byte access
+    return ((uintptr_t)(static_cast<const char*>(user) + io.off0 * 2) % 4) == 0;
+}
+
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
-                            void* stream, float* pass_ms, const ExecCallbacks* cb)
+                            void* stream, float* pass_ms, const ExecCallbacks* cb, const ExecHalf* half)
 {
     {
         const ExecPlan& chosen = select_exec_plan(plan, in, out, work, cb);
         if(&chosen != &plan)
         {
+            if(half && (half->fuse_in || half->fuse_out))
+                return rocfft_status_failure; // (decided for the primary list: the caller checks)
             // (per-pass timings describe the primary pass list: not reported for the other one)
             if(pass_ms)
                 for(size_t i = 0; i < plan.passes.size(); ++i)
@@ -2964,6 +3005,27 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
                     return rocfft_status_failure;
                 k.fast = 0;
                 k.lean = 0;
+            }
+            if(half && ((half->fuse_in && pass_index == 0) || (half->fuse_out && pass_index + 1 == npass)))
+            {
+                // the user's half array in place of the scratch copy on that side
+                if(half->fuse_in && pass_index == 0)
+                {
+                    k.in0     = static_cast<char*>(half->in) + rec.src.off0 * 2;
+                    k.in1     = static_cast<const char*>(k.in0) + 2;
+                    k.in_half = 1;
+                }
+                if(half->fuse_out && pass_index + 1 == npass)
+                {
+                    k.out0     = static_cast<char*>(half->out) + rec.dst.off0 * 2;
+                    k.out1     = static_cast<char*>(k.out0) + 2;
+                    k.out_half = 1;
+                }
+                // the other side is a scratch array of the plan (aligned)
+                if(!rec.lean_ok || with_cb || (!k.in_half && !aligned(k.in0, plan.elem_bytes))
+                   || (!k.out_half && !aligned(k.out0, plan.elem_bytes)))
+                    return rocfft_status_failure;
+                k.lean = 1;
             }
             rc = fftrt_launch_tile(&k, plan.precision, vec ? 1 : 0, rec.grid, rec.lds, stream);
         }

@@ -135,12 +135,26 @@ struct ExecCallbacks
     bool  out_complex = false;
 };
 
+// Half-precision plans compute in single precision.  Where the first (last) pass of the list is
+// a compiled kernel that converts on load (store), it reads (writes) the user's half array
+// itself; the other passes, and the sides that cannot, work on single-precision scratch arrays.
+struct ExecHalf
+{
+    void* in       = nullptr; // the user's input array of half values (interleaved or real)
+    void* out      = nullptr;
+    bool  fuse_in  = false;
+    bool  fuse_out = false;
+};
+// can the first (input = true) / last pass of the list take the user's half array at `user`?
+bool half_fusable(const ExecPlan& plan, bool input, const void* user);
+
 // Enqueues every pass on `stream`.  in/out hold one pointer (interleaved, real)
 // or two (planar).  `work` must hold plan.work_bytes() bytes when that is non-zero.
 // When pass_ms is not null every pass is bracketed by events and its duration in
 // milliseconds is written there (the call then waits for the stream).
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
-                            void* stream, float* pass_ms = nullptr, const ExecCallbacks* cb = nullptr);
+                            void* stream, float* pass_ms = nullptr, const ExecCallbacks* cb = nullptr,
+                            const ExecHalf* half = nullptr);
 
 // The pass list run_exec_plan will use for these buffers: the plan itself, or its `unaligned`
 // list when a buffer fails the alignment one of the plan's passes needs.  `work` may be null

@@ -189,6 +189,12 @@ uint32_t fftrt_fast_schedule(int precision, uint32_t n, uint32_t* radix, uint32_
     return 0;
 }
 
+// the emulation converts half-precision arrays in separate passes
+int fftrt_fast_takes_half(uint32_t)
+{
+    return 0;
+}
+
 int fftrt_launch_tile(const struct fftk_params* p, int precision, int vec, uint32_t grid,
                       size_t lds_bytes, void*)
 {

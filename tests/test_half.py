@@ -1,5 +1,8 @@
 """Half-precision plans (rocfft_precision_half): arrays of IEEE half values, arithmetic in single
-precision on staged copies.  The checker transforms the half-rounded input in long double; the
+precision.  On the GPU the first and last pass of a plan read and write the half arrays
+themselves where a compiled kernel with that form exists (interleaved or real arrays, lengths
+up to 4096 per pass); other sides go through converted copies, as everything does in the
+emulation.  The checker transforms the half-rounded input in long double; the
 result may differ by the rounding of the output to half (2^-11 relative per element)."""
 import numpy as np
 import pytest
@@ -109,5 +112,33 @@ def test_half_through_the_emulation(emu, case):
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", CASES)
 def test_half_on_the_gpu(gpu_lib, case):
+    kind, lengths, batch, kw = case
+    run_half(gpu_lib, torch_alloc, kind, lengths, batch, **kw)
+
+
+# the first and last kernel convert on load / store: one kernel, several passes (the intermediate
+# results stay in single precision), in place, short transforms (tile copy), real transforms with
+# the fused pre/post-processing, 2D/3D; and sides that fall back to converted copies (planar,
+# odd lengths, chirp-z lengths, a first pass longer than 4096 points)
+FUSED_CASES = [(B.COMPLEX_FORWARD, [4096], 64, {}), (B.COMPLEX_INVERSE, [4096], 33, {"inplace": True}),
+               (B.COMPLEX_FORWARD, [1000], 100, {}), (B.COMPLEX_FORWARD, [8], 5000, {}),
+               (B.COMPLEX_INVERSE, [16], 3001, {"inplace": True}), (B.COMPLEX_FORWARD, [65536], 5, {}),
+               (B.COMPLEX_INVERSE, [30000], 7, {"inplace": True}), (B.COMPLEX_FORWARD, [1 << 20], 1, {}),
+               (B.REAL_FORWARD, [8192], 40, {}), (B.REAL_INVERSE, [8192], 40, {}),
+               (B.REAL_FORWARD, [2000], 50, {"inplace": True}), (B.REAL_INVERSE, [2000], 50, {"inplace": True}),
+               (B.REAL_FORWARD, [32], 4000, {}), (B.REAL_INVERSE, [32], 4000, {}),
+               (B.COMPLEX_FORWARD, [256, 256], 4, {}), (B.COMPLEX_INVERSE, [100, 60], 9, {"inplace": True}),
+               (B.REAL_FORWARD, [512, 512], 3, {}), (B.REAL_INVERSE, [512, 512], 3, {}),
+               (B.COMPLEX_FORWARD, [64, 64, 64], 2, {}), (B.REAL_FORWARD, [48, 40, 36], 2, {}),
+               (B.REAL_INVERSE, [48, 40, 36], 2, {"inplace": True}), (B.COMPLEX_FORWARD, [4, 5], 3000, {}),
+               (B.COMPLEX_FORWARD, [360, 360], 2, {"planar": True}), (B.REAL_FORWARD, [1001], 20, {}),
+               (B.REAL_INVERSE, [625], 20, {}), (B.COMPLEX_FORWARD, [173], 100, {}),
+               (B.COMPLEX_FORWARD, [8192], 10, {}), (B.REAL_FORWARD, [65536], 6, {}),
+               (B.REAL_INVERSE, [65536], 6, {})]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", FUSED_CASES)
+def test_half_arrays_read_and_written_by_the_kernels(gpu_lib, case):
     kind, lengths, batch, kw = case
     run_half(gpu_lib, torch_alloc, kind, lengths, batch, **kw)
