@@ -2576,6 +2576,12 @@ static rocfft_status build_exec_plan_once(const Problem& p, ExecPlan& plan, bool
             uint64_t half = n0 / 2;
             View     rv   = realpair_view(out_buf, p.ostride, p.odist, p.ooffset, p.rank);
             auto     oth  = other_axes(hv, rv, p.len, p.rank, p.batch, 0);
+            // in place with the standard padded rows (the real row of a bin row starts where the bin
+            // row starts): the pre-processing step can run in place and leave the half-length
+            // transform to whatever plan suits that length, as out of place
+            bool standard_inplace = plan.inplace && !hv.io.planar && hv.stride[0] == rv.stride[0] && rv.io.im_delta == 1;
+            for(int d = 1; d < 4; ++d)
+                standard_inplace = standard_inplace && hv.stride[d] == rv.stride[d];
             if(half == 1)
             {
                 // two real samples a row: the pre-processing step alone, from the input bins to the
@@ -2589,7 +2595,7 @@ static rocfft_status build_exec_plan_once(const Problem& p, ExecPlan& plan, bool
             else if(big_eligible(b, half, hv.stride[0], rv.stride[0], oth, hv.io, rv.io))
                 emit_big(b, 2, oth, hv.io, rv.io, +1, p.scale, p.has_scale);
             else if(single_kernel_length(half, b.esize)
-                    && (plan.inplace
+                    && ((plan.inplace && !standard_inplace)
                         || plain_dim_is_single(half, rv.stride[0] != 2, b.esize, hv.stride[0], rv.stride[0])))
             {
                 // (out of place, a half length that only the run-time-schedule kernel takes in one

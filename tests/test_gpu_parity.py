@@ -215,6 +215,20 @@ def test_real_rows_of_two_samples(gpu):
         H.check(lib, be, K.REAL_INVERSE, lengths, batch, K.SINGLE, in_type=K.HERMITIAN_PLANAR, scale=2.0)
 
 
+def test_in_place_real_inverse_without_a_compiled_half_length(gpu):
+    """In place, with the standard padded rows, a real inverse transform whose half length has no
+    compiled kernel in that precision runs the pre-processing step in place and then the same
+    passes as out of place (it used to run one run-time-schedule kernel)."""
+    lib, be = gpu
+    st, text, _ = lib.describe(B.INPLACE, B.REAL_INVERSE, B.DOUBLE, [11200], 8)
+    assert st == 0 and "real pre-process" in text and "split" in text, text
+    for n in (11200, 9000, 10000):
+        H.check(lib, be, B.REAL_INVERSE, [n], 5, B.DOUBLE, inplace=True)
+        H.check(lib, be, B.REAL_INVERSE, [n], 3, B.DOUBLE, inplace=True, scale=0.5)
+        H.check(lib, be, B.REAL_FORWARD, [n], 3, B.DOUBLE, inplace=True)
+    H.check(lib, be, B.REAL_INVERSE, [11200, 6], 2, B.DOUBLE, inplace=True)
+
+
 def test_column_tiles_that_span_more_than_two_gib(gpu):
     """A column pass whose tile reaches from the first to the last byte of a 2 GiB array: element
     offsets inside the tile need 29 bits in single precision (129 x 2^21 elements), byte offsets 32."""
