@@ -10,9 +10,10 @@ of place, through rocfft_execute of this library's C ABI.
 Prints ONE JSON line.  `value` is GFLOP/s in the 5*N*log2(N) convention summed
 over the transforms of a step.  `roofline` prices the slowest kernel of the step
 against the HBM peak using per-kernel durations taken with HIP events inside this
-script; `cpu_baseline` times the CPU checker (a port of the algorithm, OpenMP
-across the batch) on a bounded sample of the same workload; `cpu_other` adds what
-else the host offers (FFTW or MKL when a dlopen finds them, scipy's pocketfft).
+script; `cpu_baseline` is the fastest CPU figure the host offers for a bounded sample
+of the same workload, looked for in the order FFTW (the reference's CPU path), MKL's
+FFTW interface, scipy's pocketfft, this repository's own port (`kind` and `chain` say
+which was found and used); `cpu_other` holds the remaining ones.
 `all_configs` adds one short measurement for each of the five benchmark
 configurations next to reference rocFFT, timed through the identical harness (the
 same rocfft.h calls on the same buffers, preallocated outputs, caller-owned work
@@ -155,10 +156,8 @@ def kernel_profile(step, reps):
     return acc
 
 
-def cpu_baseline(cfg_id, wl, budget_s=12.0):
+def cpu_port(cfg_id, wl, budget_s=6.0):
     """the CPU checker (double precision port, OpenMP over the batch) on a bounded sample"""
-    import numpy as np
-
     import inputs
     from oracle import oracle as orc
 
@@ -187,6 +186,103 @@ def cpu_baseline(cfg_id, wl, budget_s=12.0):
     return dict(value=wl["flops"] * frac / t / 1e9, unit="GFLOP/s", cores=threads, kind="port",
                 sample="%d of %d transforms of %s, %.1f s, oracle/fft_oracle.c double build, %d OpenMP threads"
                 % (nb, full_batch, "x".join(map(str, lengths)), t, threads))
+
+
+def host_threads():
+    """threads for the CPU baselines: the CPUs this process may run on (the reference's tests
+    size FFTW's thread pool the same way, shared/concurrency.h:33-41), at most 16"""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        n = os.cpu_count() or 1
+    return max(1, min(16, n))
+
+
+def cpu_pocketfft(cfg_id, wl, budget_s=10.0, min_s=1.0):
+    """scipy.fft (pocketfft, C++) on the same workload in the workload's own precision: batched
+    contiguous out-of-place transforms, `workers` threads across the batch, planning (pocketfft
+    caches its plans after the first call) outside the timed repetitions.  The sample is at
+    least 1024 signals of the batched workloads and is repeated for at least min_s seconds."""
+    import numpy as np
+    import scipy.fft as sf
+
+    import inputs
+
+    threads = host_threads()
+    full = wl["transforms"][0][2]
+    lengths = wl["transforms"][0][1]
+    nb = {1: 1024, 2: 1024, 3: 2, 4: 1, 5: 16}[cfg_id]
+    x = inputs.config_input(cfg_id, 0, nb)
+    if cfg_id in (1, 3):
+        x = x.astype(np.complex64)
+    elif cfg_id == 2:
+        x = x.astype(np.float32)
+    if cfg_id == 3:
+        x = x.reshape(nb, 4096, 4096)
+    elif cfg_id == 4:
+        x = x.reshape(512, 512, 512)
+
+    def run():
+        if cfg_id == 2:
+            return sf.irfft(sf.rfft(x, axis=1, workers=threads), n=65536, axis=1, workers=threads)
+        if cfg_id == 3:
+            return sf.fft2(x, axes=(1, 2), workers=threads)
+        if cfg_id == 4:
+            return sf.irfftn(sf.rfftn(x, workers=threads), s=(512, 512, 512), workers=threads)
+        return sf.fft(x, axis=1, workers=threads)
+
+    run()
+    ts = []
+    t_all = time.perf_counter()
+    while (time.perf_counter() - t_all < min_s or len(ts) < 3) and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
+        run()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    t = ts[len(ts) // 2]
+    return dict(value=wl["flops"] * (nb / full) / t / 1e9, unit="GFLOP/s", cores=threads,
+                kind="library: scipy.fft (pocketfft) %s, %s" % (x.dtype, "rfft + irfft" if cfg_id in (2, 4) else "fft"),
+                sample="%d of %d transforms of %s, median of %d repetitions of %.3f s (%.1f s in all), %d workers"
+                % (nb, full, "x".join(map(str, lengths)), len(ts), t, sum(ts), threads))
+
+
+def cpu_baseline(cfg_id, wl):
+    """The fastest CPU figure this machine offers, in the order the reference's own tests would
+    find one: FFTW (the reference's CPU path, clients/tests/CMakeLists.txt:128-129), MKL's FFTW
+    interface, scipy's pocketfft, this repository's port.  `chain` records what each probe found;
+    the others are reported under cpu_other."""
+    import ctypes
+
+    chain = {}
+    for name in ("libfftw3f.so.3", "libfftw3.so.3", "libfftw3f_threads.so.3", "libfftw3f_omp.so.3", "libmkl_rt.so",
+                 "libmkl_rt.so.2"):
+        try:
+            ctypes.CDLL(name)
+            chain[name] = True
+        except OSError:
+            chain[name] = False
+    cands = {}
+    if cfg_id == 2 and chain.get("libfftw3f.so.3"):
+        try:
+            cands["fftw"] = fftw_r2c_c2r(wl)
+        except Exception as e:  # noqa: BLE001
+            cands["fftw"] = {"error": repr(e)[:200]}
+    try:
+        cands["pocketfft"] = cpu_pocketfft(cfg_id, wl)
+    except Exception as e:  # noqa: BLE001
+        cands["pocketfft"] = {"error": repr(e)[:200]}
+    try:
+        cands["port"] = cpu_port(cfg_id, wl)
+    except Exception as e:  # noqa: BLE001
+        cands["port"] = {"error": repr(e)[:200]}
+    ok = {k: v for k, v in cands.items() if "value" in v}
+    # FFTW when present (it is the reference's own CPU path), else the fastest of the others
+    pick = "fftw" if "fftw" in ok else max(ok, key=lambda k: ok[k]["value"])
+    base = dict(ok[pick])
+    base["chain"] = chain
+    other = {k: v for k, v in cands.items() if k != pick}
+    other["dlopen"] = chain
+    return base, other
 
 
 def torch_fft_ms(torch, cfg_id, step, reps=5):
@@ -287,61 +383,7 @@ def reference_rocfft(warmup, steps, timeout_s=240):
     return results
 
 
-def cpu_other(cfg_id, wl, budget_s=6.0):
-    """what else the host offers for the same workload: the reference's CPU path is FFTW
-    (clients/tests/CMakeLists.txt:128-129), looked for with dlopen together with MKL's FFTW
-    interface; scipy's pocketfft (threads stated) is timed in any case.  Configuration 2 only."""
-    import ctypes
-
-    import numpy as np
-
-    found = {}
-    for name in ("libfftw3f.so.3", "libfftw3.so.3", "libfftw3f_threads.so.3", "libfftw3f_omp.so.3", "libmkl_rt.so",
-                 "libmkl_rt.so.2"):
-        try:
-            ctypes.CDLL(name)
-            found[name] = True
-        except OSError:
-            found[name] = False
-    out = {"dlopen": found}
-    if cfg_id != 2:
-        return out
-    import inputs
-
-    n, full = 65536, 4096
-    threads = min(16, os.cpu_count() or 1)
-    nb = 256
-    x = inputs.config_input(2, 0, nb).astype(np.float32)
-    try:
-        import scipy.fft as sf
-
-        def run():
-            return sf.irfft(sf.rfft(x, axis=1, workers=threads), n=n, axis=1, workers=threads)
-
-        run()
-        t0 = time.perf_counter()
-        reps = 0
-        while time.perf_counter() - t0 < budget_s and reps < 20:
-            run()
-            reps += 1
-        t = (time.perf_counter() - t0) / reps
-        out["pocketfft"] = dict(value=wl["flops"] * (nb / full) / t / 1e9, unit="GFLOP/s", cores=threads,
-                                kind="scipy.fft (pocketfft) float32, rfft + irfft",
-                                sample="%d of %d transforms of %d, %.2f s per repetition, %d workers"
-                                % (nb, full, n, t, threads))
-    except Exception as e:  # noqa: BLE001
-        out["pocketfft"] = {"error": repr(e)[:200]}
-    if found.get("libfftw3f.so.3"):
-        try:
-            out["fftw"] = fftw_r2c_c2r(x, n, nb, wl, full, budget_s)
-        except Exception as e:  # noqa: BLE001
-            out["fftw"] = {"error": repr(e)[:200]}
-    else:
-        out["fftw"] = None  # not installed on this machine
-    return out
-
-
-def fftw_r2c_c2r(x, n, nb, wl, full, budget_s):
+def fftw_r2c_c2r(wl, budget_s=10.0, min_s=1.0):
     """FFTW single precision, batched contiguous out-of-place plans with FFTW_ESTIMATE as the
     reference's tests make them (shared/rocfft_against_fftw.h:108-142); one thread unless the
     threads library is present"""
@@ -349,13 +391,17 @@ def fftw_r2c_c2r(x, n, nb, wl, full, budget_s):
 
     import numpy as np
 
+    import inputs
+
+    n, full, nb = 65536, 4096, 1024
+    x = inputs.config_input(2, 0, nb).astype(np.float32)
     fw = ctypes.CDLL("libfftw3f.so.3")
     threads = 1
     for tl in ("libfftw3f_omp.so.3", "libfftw3f_threads.so.3"):
         try:
             ft = ctypes.CDLL(tl, mode=ctypes.RTLD_GLOBAL)
             ft.fftwf_init_threads()
-            threads = min(16, os.cpu_count() or 1)
+            threads = host_threads()
             ft.fftwf_plan_with_nthreads(threads)
             break
         except (OSError, AttributeError):
@@ -374,15 +420,106 @@ def fftw_r2c_c2r(x, n, nb, wl, full, budget_s):
     if not pf or not pb:
         raise RuntimeError("fftwf_plan_many_dft failed")
     fw.fftwf_execute.argtypes = [ctypes.c_void_p]
-    t0 = time.perf_counter()
-    reps = 0
-    while time.perf_counter() - t0 < budget_s and reps < 20:
+    ts = []
+    t_all = time.perf_counter()
+    while (time.perf_counter() - t_all < min_s or len(ts) < 3) and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
         fw.fftwf_execute(pf)
         fw.fftwf_execute(pb)
-        reps += 1
-    t = (time.perf_counter() - t0) / reps
-    return dict(value=wl["flops"] * (nb / full) / t / 1e9, unit="GFLOP/s", cores=threads, kind="FFTW 3 float32",
-                sample="%d of %d transforms of %d, %.2f s per repetition" % (nb, full, n, t))
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    t = ts[len(ts) // 2]
+    return dict(value=wl["flops"] * (nb / full) / t / 1e9, unit="GFLOP/s", cores=threads,
+                kind="reference: FFTW 3 float32, FFTW_ESTIMATE",
+                sample="%d of %d transforms of %d, median of %d repetitions of %.3f s" % (nb, full, n, len(ts), t))
+
+
+def copy_probes():
+    """name -> fields of rocfft_amd_copy_probe: plain copies of 1 GiB in the access shapes of the
+    passes of the five configurations (element = 8 bytes unless said)"""
+    import rocfft_amd.binding as B
+
+    gib = 1 << 30
+    rows = 4096  # rows of 32768 elements of 8 bytes: 1 GiB
+    tiles = dict(shape=B.PROBE_TILES, rows=0, tile_width=64, elem_bytes=8)
+    return {
+        "stream, 16 B per lane, 4 workgroups per CU": dict(shape=B.PROBE_STREAM, bytes=gib),
+        "stream, nontemporal": dict(shape=B.PROBE_STREAM, bytes=gib, nontemporal=1),
+        "stream, 8 workgroups per CU": dict(shape=B.PROBE_STREAM, bytes=gib, workgroups_per_cu=8),
+        "stream, 64 workgroups per CU": dict(shape=B.PROBE_STREAM, bytes=gib, workgroups_per_cu=64),
+        "read only": dict(shape=B.PROBE_READ, bytes=gib),
+        "write only": dict(shape=B.PROBE_WRITE, bytes=gib),
+        # configuration 2: one workgroup of 1024 threads per row of 256 KiB
+        "rows of 32768, 32 loads then 32 stores, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=32, workgroups_per_cu=1),
+        "rows of 32768, 8 loads then 8 stores, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=8, workgroups_per_cu=1),
+        "rows of 32768 read, rows 32769 apart written (real forward), 32/32": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32769, group=32, workgroups_per_cu=1),
+        "rows 32769 apart read, rows of 32768 written (real inverse), 32/32": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32769, out_row=32768, group=32, workgroups_per_cu=1),
+        "rows 32769 apart written, 8/8": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32769, group=8, workgroups_per_cu=1),
+        "rows 32769 apart written, 32/32, 2 workgroups per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32769, group=32, workgroups_per_cu=2),
+        # configurations 1 and 3, row pass: a tile is one contiguous row of 4096 elements
+        "tiles 4096 x 1 (contiguous rows of 32 KiB), one workgroup per tile": dict(tiles, tile_width=256, in_row=256, out_row=256, tiles_per_slab=1, rows=32768, in_slab=4096, out_slab=4096),
+        "tiles 4096 x 1, nontemporal": dict(tiles, tile_width=256, in_row=256, out_row=256, tiles_per_slab=1, rows=32768, in_slab=4096, out_slab=4096, nontemporal=1),
+        "tiles 4096 x 1, resident grid": dict(tiles, tile_width=256, in_row=256, out_row=256, tiles_per_slab=1, rows=32768, in_slab=4096, out_slab=4096, resident_grid=1),
+        # configuration 3, column passes: 64 columns x 64 rows, rows 4128 elements apart
+        "tiles 64 x 64, rows 4128 apart (configuration 3, column passes)": dict(tiles, in_row=4128, out_row=4128, tiles_per_slab=64, rows=512, in_slab=64 * 4128, out_slab=64 * 4128),
+        "tiles 64 x 64, rows 4128 apart, nontemporal": dict(tiles, in_row=4128, out_row=4128, tiles_per_slab=64, rows=512, in_slab=64 * 4128, out_slab=64 * 4128, nontemporal=1),
+        "tiles 64 x 64, rows 4128 apart, resident grid": dict(tiles, in_row=4128, out_row=4128, tiles_per_slab=64, rows=512, in_slab=64 * 4128, out_slab=64 * 4128, resident_grid=1),
+        "tiles 64 x 64, rows 4096 apart (power-of-two pitch)": dict(tiles, in_row=4096, out_row=4096, tiles_per_slab=64, rows=512, in_slab=64 * 4096, out_slab=64 * 4096),
+        # configuration 4, column passes: 8 columns of 16 bytes x 512 rows
+        "tiles 8 x 512 of 16 B, rows 257 apart (configuration 4, y columns)": dict(tiles, tile_width=8, elem_bytes=16, in_row=257, out_row=257, tiles_per_slab=32, rows=512, in_slab=257 * 512, out_slab=257 * 512),
+        "tiles 8 x 512 of 16 B, rows 131584 apart (configuration 4, z columns)": dict(tiles, tile_width=8, elem_bytes=16, in_row=131584, out_row=131584, tiles_per_slab=16384, rows=1, in_slab=0, out_slab=0),
+        "tiles 8 x 512 of 16 B, rows 131584 apart, nontemporal": dict(tiles, tile_width=8, elem_bytes=16, in_row=131584, out_row=131584, tiles_per_slab=16384, rows=1, in_slab=0, out_slab=0, nontemporal=1),
+        "tiles 16 x 256 of 16 B, rows 131584 apart": dict(tiles, tile_width=16, elem_bytes=16, in_row=131584, out_row=131584, tiles_per_slab=8192, rows=2, in_slab=131584 * 256, out_slab=131584 * 256),
+    }
+
+
+def copy_ceilings(torch, lib, names=None, reps=10):
+    """name -> (median ms, TB/s counting bytes read + bytes written) of the copy probes"""
+    import rocfft_amd.binding as B
+
+    dev = torch.device("cuda:0")
+    src = torch.rand((1 << 28) + (1 << 22), dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    stream_ptr = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for name, f in copy_probes().items():
+        if names is not None and name not in names:
+            continue
+        f = dict(f, src=src.data_ptr(), dst=dst.data_ptr())
+        if f["shape"] == B.PROBE_ROWS:
+            moved = 2.0 * f["rows"] * 32768 * 8
+        elif f["shape"] == B.PROBE_TILES:
+            moved = 2.0 * f["tiles_per_slab"] * f["rows"] * 4096 * f["elem_bytes"]
+        elif f["shape"] == B.PROBE_STREAM:
+            moved = 2.0 * f["bytes"]
+        else:
+            moved = 1.0 * f["bytes"]
+        for _ in range(2):
+            lib.copy_probe(stream_ptr, **f)
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            lib.copy_probe(stream_ptr, **f)
+            b.record()
+            torch.cuda.synchronize()
+            ts.append(a.elapsed_time(b))
+        ts.sort()
+        ms = ts[len(ts) // 2]
+        out[name] = (ms, moved / (ms * 1e-3) / 1e12)
+    return out
+
+
+# the copy probe whose access shape is that of the slowest kernel of a configuration
+SHAPE_OF_CONFIG = {
+    1: "tiles 4096 x 1 (contiguous rows of 32 KiB), one workgroup per tile",
+    2: "rows 32769 apart read, rows of 32768 written (real inverse), 32/32",
+    3: "tiles 64 x 64, rows 4128 apart (configuration 3, column passes)",
+    4: "tiles 8 x 512 of 16 B, rows 131584 apart (configuration 4, z columns)",
+    5: "tiles 4096 x 1 (contiguous rows of 32 KiB), one workgroup per tile",
+}
 
 
 def measure_config(torch, cfg_id, wl, stream_ptr, warmup, steps, prof_reps):
@@ -402,6 +539,9 @@ def main():
     ap.add_argument("--reference-lib", default=None,
                     help="(used by this script for its child processes) time the five configurations on the "
                          "rocfft.h library at this path and print them as JSON")
+    ap.add_argument("--copy-ceilings", action="store_true",
+                    help="time plain copies of 1 GiB in the access shapes of the passes (rocfft_amd_copy_probe) and "
+                         "print them as a table: what the memory system gives a copy of each shape")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain elementwise copy of 1 GiB (reads 1 GiB, writes 1 GiB) ten times: "
                          "the known-size kernel the rocprofv3 FETCH_SIZE/WRITE_SIZE counters are scaled by")
@@ -415,7 +555,7 @@ def main():
     # the reference library's figures come from child processes, started before this process
     # initialises the GPU
     refs = []
-    if not (args.no_extras or args.reference_lib or args.calibrate_copy):
+    if not (args.no_extras or args.reference_lib or args.calibrate_copy or args.copy_ceilings):
         refs = reference_rocfft(2, 10)
 
     import torch
@@ -438,7 +578,15 @@ def main():
         print(json.dumps({"calibration": "torch.mul(src, 1.0, out=dst), float32", "bytes_read": 4 * n,
                           "bytes_written": 4 * n, "launches": 10}))
         return
-    rf.library()  # raises if the HIP library is not built
+    lib = rf.library()  # raises if the HIP library is not built
+    if args.copy_ceilings:
+        res = copy_ceilings(torch, lib)
+        print("| copy of 1 GiB (1 GiB read, 1 GiB written unless said) | ms | TB/s | of 8 TB/s |")
+        print("|---|---|---|---|")
+        for name, (ms, tbs) in res.items():
+            print("| %s | %.3f | %.2f | %.3f |" % (name, ms, tbs, tbs * 1e3 / HBM_PEAK_GBS))
+        print(json.dumps({"copy_ceilings_TBps": {k: v[1] for k, v in res.items()}}))
+        return
     stream_ptr = torch.cuda.current_stream().cuda_stream
     wls = workloads()
     wl = wls[args.config]
@@ -453,6 +601,14 @@ def main():
             traffic = json.load(open(tpath)).get(wl["name"], {}).get(dom[0])
         except Exception:  # noqa: BLE001
             traffic = None
+    # the same kernel against a plain copy in its access shape, and against the best copy seen
+    shape = SHAPE_OF_CONFIG[args.config]
+    best = "stream, nontemporal"
+    try:
+        cc = copy_ceilings(torch, lib, names={shape, best})
+        copy_shape, copy_best = cc[shape][1] * 1e3, cc[best][1] * 1e3
+    except Exception:  # noqa: BLE001
+        copy_shape = copy_best = None
     out = {
         "metric": "GFLOP/s (5N*log2N) per config, 1 GPU",
         "value": wl["flops"] / (ms * 1e-3) / 1e9,
@@ -473,7 +629,10 @@ def main():
         "algorithmic_hbm_frac": wl["bytes"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": dom[0],
-                     "kernel_ms": dom[2], "kernel_bytes": dom[1]},
+                     "kernel_ms": dom[2], "kernel_bytes": dom[1],
+                     "frac_of_copy": achieved / copy_shape if copy_shape else None,
+                     "copy_of_shape_GBps": copy_shape, "copy_shape": shape,
+                     "best_copy_GBps": copy_best},
         "kernels": [{"name": n, "bytes": b, "ms": t, "GBps": b / (t * 1e-3) / 1e9 if t > 0 else None}
                     for n, b, t in prof],
     }
@@ -509,8 +668,7 @@ def main():
         out["reference_rocfft"] = refs
         del step
         torch.cuda.empty_cache()
-        out["cpu_baseline"] = cpu_baseline(args.config, wl)
-        out["cpu_other"] = cpu_other(args.config, wl)
+        out["cpu_baseline"], out["cpu_other"] = cpu_baseline(args.config, wl)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

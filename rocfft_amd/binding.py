@@ -39,7 +39,8 @@ class RocfftError(RuntimeError):
 
 
 def library_path():
-    return os.path.join(_HERE, "lib", "librocfft_amd.so")
+    """the product library; ROCFFT_AMD_LIBRARY names another build of it (experiments)"""
+    return os.environ.get("ROCFFT_AMD_LIBRARY") or os.path.join(_HERE, "lib", "librocfft_amd.so")
 
 
 _c_size_p = ctypes.POINTER(ctypes.c_size_t)
@@ -91,7 +92,21 @@ _PROTOTYPES = {
     "rocfft_amd_execute_profile": [ctypes.c_void_p, _c_void_pp, _c_void_pp, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_float), ctypes.c_size_t],
     "rocfft_amd_execute_static": [ctypes.c_void_p, _c_void_pp, _c_void_pp, ctypes.c_void_p],
+    "rocfft_amd_copy_probe": [ctypes.c_void_p, ctypes.c_void_p],
 }
+
+
+class Probe(ctypes.Structure):
+    """rocfft_amd_probe of include/rocfft_amd.h: one plain copy in the access shape of a pass"""
+    _fields_ = [("shape", ctypes.c_int), ("src", ctypes.c_void_p), ("dst", ctypes.c_void_p),
+                ("bytes", ctypes.c_size_t), ("nontemporal", ctypes.c_int), ("workgroups_per_cu", ctypes.c_uint),
+                ("group", ctypes.c_uint), ("rows", ctypes.c_uint), ("in_row", ctypes.c_size_t),
+                ("out_row", ctypes.c_size_t), ("tile_width", ctypes.c_uint), ("elem_bytes", ctypes.c_uint),
+                ("tiles_per_slab", ctypes.c_uint), ("in_slab", ctypes.c_size_t), ("out_slab", ctypes.c_size_t),
+                ("resident_grid", ctypes.c_int)]
+
+
+PROBE_STREAM, PROBE_READ, PROBE_WRITE, PROBE_ROWS, PROBE_TILES = range(5)
 
 # size of the device-resident work area behind rocfft_amd_execute_static
 STATIC_WORK_BYTES = 64 << 20
@@ -142,6 +157,11 @@ class Library:
         buf = ctypes.create_string_buffer(64)
         self.check(self.c.rocfft_get_version_string(buf, 64), "rocfft_get_version_string")
         return buf.value.decode()
+
+    def copy_probe(self, stream=None, **fields):
+        """enqueues one copy probe (rocfft_amd_copy_probe) on `stream`"""
+        q = Probe(**fields)
+        self.check(self.c.rocfft_amd_copy_probe(ctypes.byref(q), stream), "rocfft_amd_copy_probe")
 
     def describe(self, placement, transform_type, precision, lengths, batch=1, description=None):
         """Plan text and work-buffer bytes without touching a device."""

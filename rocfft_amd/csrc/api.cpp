@@ -38,31 +38,20 @@ struct rocfft_plan_description_t
 
 // Device buffers a plan keeps for executions that stage through copies (load/store callbacks,
 // half precision): the copies of the input and output arrays and, when the caller sets no work
-// buffer, the work area.  One set per stream the plan has been executed on, allocated by the
-// first such execution on that stream and released with the plan, so that later executions
-// allocate nothing, do not wait for the stream and can be captured into a graph.
+// buffer, the work area.  One set per stream the plan has been executed on.  A buffer is
+// allocated by the first execution on that stream that needs it and replaced by a larger one
+// when a later execution needs more; nothing is freed before the plan is destroyed (a graph
+// captured earlier, or a thread that has read the pointers and not yet enqueued its kernels,
+// may still use a replaced buffer), so that executions which find what they need allocate
+// nothing, do not wait for the stream and can be captured into a graph.
+struct StageBuf
+{
+    void*  ptr   = nullptr;
+    size_t bytes = 0;
+};
 struct StageSet
 {
-    void*  in[2]    = {nullptr, nullptr};
-    void*  out[2]   = {nullptr, nullptr};
-    void*  work     = nullptr;
-    size_t in_bytes = 0, out_bytes = 0, work_bytes = 0;
-    bool   shared   = false; // in-place: out[] are in[]
-    void   release()
-    {
-        for(int i = 0; i < 2; ++i)
-        {
-            if(out[i] && !shared)
-                fftrt_free(out[i]);
-            if(in[i])
-                fftrt_free(in[i]);
-            in[i] = out[i] = nullptr;
-        }
-        if(work)
-            fftrt_free(work);
-        work     = nullptr;
-        in_bytes = out_bytes = work_bytes = 0;
-    }
+    StageBuf in[2], out[2], work;
 };
 
 struct rocfft_plan_t
@@ -72,14 +61,30 @@ struct rocfft_plan_t
     int         device = 0;
     std::string error;
     bool        half_io = false; // half-precision arrays: the plan computes in single precision on scratch copies
+    // stage_lock is held from the lookup of a set until every kernel that uses its buffers has
+    // been enqueued: the order of enqueueing on a stream is then the order of use
     std::mutex                stage_lock;
     std::map<void*, StageSet> stage; // by stream
+    std::vector<void*>        stage_allocs; // every buffer of every set, replaced ones included
+    // makes b hold at least `bytes`; false when the allocation fails
+    bool stage_grow(StageBuf& b, size_t bytes)
+    {
+        if(b.ptr && b.bytes >= bytes)
+            return true;
+        void* p = nullptr;
+        if(fftrt_malloc(&p, bytes) != 0)
+            return false;
+        stage_allocs.push_back(p);
+        b.ptr   = p;
+        b.bytes = bytes;
+        return true;
+    }
     ~rocfft_plan_t()
     {
-        if(!stage.empty())
+        if(!stage_allocs.empty())
             fftrt_device_sync(); // executions in flight may still use the buffers
-        for(auto& kv : stage)
-            kv.second.release();
+        for(void* p : stage_allocs)
+            fftrt_free(p);
     }
 };
 
@@ -488,6 +493,13 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         if((planar(pr.in_type) && !in[1]) || (planar(pr.out_type) && !out[1]))
             return rocfft_status_failure;
         void*  stream = info ? info->stream : nullptr;
+        // the work area the pass-list choice is made for: the library's static array when that
+        // will be used, else the caller's buffer (null: an aligned allocation follows)
+        void*  static_ptr  = nullptr;
+        size_t static_have = 0;
+        if(static_work && fftrt_static_scratch(&static_ptr, &static_have) != 0)
+            return rocfft_status_failure;
+        void* const work_hint = static_work ? static_ptr : (info ? info->workBuffer : nullptr);
         // Load/store callbacks run inside the first and last kernel when those have a callback
         // form (interleaved or real arrays); otherwise, and for half precision, the arrays are
         // staged through copies.
@@ -503,30 +515,27 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
             ecb.store_data  = info->store_cb_data;
             ecb.in_complex  = pr.in_type != rocfft_array_type_real;
             ecb.out_complex = pr.out_type != rocfft_array_type_real;
-            fused           = callbacks_fusable(ep, in, out, info->workBuffer, ecb);
+            fused           = callbacks_fusable(ep, in, out, work_hint, ecb);
         }
         const bool staging = half_io || (have_cb && !fused);
+        if(staging && have_cb && (planar(pr.in_type) || planar(pr.out_type) || half_io))
+            return rocfft_status_failure;
         // the work area of the pass list these buffers get (staged copies are aligned allocations)
         size_t need = staging ? ep.work_bytes()
-                              : select_exec_plan(ep, in, out, info ? info->workBuffer : nullptr, fused ? &ecb : nullptr)
-                                    .own_work_bytes();
-        if(staging && static_work)
-            return rocfft_status_failure; // staged copies live in buffers the plan allocates
+                              : select_exec_plan(ep, in, out, work_hint, fused ? &ecb : nullptr).own_work_bytes();
         void* work = nullptr;
         bool  own  = false;
         if(need && static_work)
         {
-            size_t have = 0;
-            if(fftrt_static_scratch(&work, &have) != 0)
-                return rocfft_status_failure;
-            if(need > have)
+            if(need > static_have)
             {
                 fprintf(stderr,
                         "rocfft_amd_execute_static: the plan needs %zu bytes of work area, the static area "
                         "holds %zu\n",
-                        need, have);
+                        need, static_have);
                 return rocfft_status_invalid_work_buffer;
             }
+            work = static_ptr;
         }
         else if(need)
         {
@@ -557,13 +566,14 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
             }
         };
 
-        // Staging.  Load/store callbacks: the input is copied into a scratch buffer of the same
-        // layout through the load callback, the plan runs on scratch buffers, and the result
-        // goes to the user's buffer through the store callback (two extra element-wise
-        // passes; the transform kernels themselves make no indirect calls).  Half precision:
-        // the plan computes in single precision on scratch arrays of the same layout, filled
-        // from and written back to the user's half-precision arrays the same way.  The scratch
-        // arrays belong to the plan (one set per stream, see StageSet).
+        // Staging.  Load/store callbacks no kernel of the pass list can call: the input is copied
+        // into a scratch buffer of the same layout through the load callback, the plan runs on
+        // scratch buffers, and the result goes to the user's buffer through the store callback.
+        // Half precision: the plan computes in single precision; a first (last) pass that converts
+        // on load (store) takes the user's half array itself, every other access to the input
+        // (output) array goes to a single-precision scratch array of the same layout, which a
+        // copy fills from (writes back to) the user's array when the pass on that side cannot
+        // convert.  The scratch arrays belong to the plan (one set per stream, see StageSet).
         void*          st_in[2]  = {nullptr, nullptr};
         void*          st_out[2] = {nullptr, nullptr};
         fftk_cb_params cin, cout;
@@ -574,12 +584,12 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
         const bool in_complex  = pr.in_type != rocfft_array_type_real && !in_planar;
         const bool out_complex = pr.out_type != rocfft_array_type_real && !out_planar;
         const int  nin = in_planar ? 2 : 1, nout = out_planar ? 2 : 1;
-        bool       stage_in = false, stage_out = false;
+        bool       stage_in = false, stage_out = false; // that side has a scratch array
+        bool       copy_in = false, copy_out = false;   // ... which a separate pass fills / writes back
         ExecHalf   ehalf;
+        std::unique_lock<std::mutex> stage_guard(plan->stage_lock, std::defer_lock);
         if(staging)
         {
-            if(have_cb && (in_planar || out_planar || half_io))
-                return rocfft_status_failure;
             const size_t scalar = ep.precision ? 8 : 4; // of the scratch arrays
             auto         fill   = [&](fftk_cb_params& c, bool input) {
                 size_t off0   = input ? std::max(pr.ioffset[0], pr.ioffset[1]) : std::max(pr.ooffset[0], pr.ooffset[1]);
@@ -601,75 +611,69 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
             };
             size_t       in_bytes  = fill(cin, true);
             const size_t out_bytes = fill(cout, false);
-            stage_in               = ep.inplace || half_io || info->load_cb;
-            stage_out              = ep.inplace || half_io || info->store_cb;
             if(ep.inplace)
                 in_bytes = std::max(in_bytes, out_bytes);
-            const size_t want_work = (need && !work) ? need : 0;
-            {
-                std::lock_guard<std::mutex> guard(plan->stage_lock);
-                StageSet&                   set = plan->stage[stream];
-                const bool fits = (!stage_in || (set.in[0] && set.in_bytes >= in_bytes && (nin < 2 || set.in[1])))
-                                  && (!stage_out || ep.inplace
-                                      || (set.out[0] && set.out_bytes >= out_bytes && (nout < 2 || set.out[1])))
-                                  && (!ep.inplace || set.shared || !set.in[0])
-                                  && set.work_bytes >= want_work;
-                if(!fits)
-                {
-                    // (re)allocate: not while the stream is being captured, and only after
-                    // earlier executions on this stream have let go of the old buffers
-                    if(fftrt_stream_capturing(stream))
-                        return rocfft_status_failure;
-                    fftrt_stream_sync(stream);
-                    set.release();
-                    bool ok = true;
-                    for(int i = 0; i < nin && ok && stage_in; ++i)
-                        ok = fftrt_malloc(&set.in[i], in_bytes) == 0;
-                    set.in_bytes = stage_in ? in_bytes : 0;
-                    set.shared   = ep.inplace;
-                    for(int i = 0; i < nout && ok && stage_out; ++i)
-                    {
-                        if(ep.inplace)
-                            set.out[i] = set.in[i];
-                        else
-                            ok = fftrt_malloc(&set.out[i], out_bytes) == 0;
-                    }
-                    set.out_bytes = stage_out ? (ep.inplace ? in_bytes : out_bytes) : 0;
-                    if(ok && want_work)
-                    {
-                        ok             = fftrt_malloc(&set.work, want_work) == 0;
-                        set.work_bytes = ok ? want_work : 0;
-                    }
-                    if(!ok)
-                    {
-                        set.release();
-                        return rocfft_status_failure;
-                    }
-                }
-                for(int i = 0; i < 2; ++i)
-                {
-                    st_in[i]  = stage_in ? set.in[i] : nullptr;
-                    st_out[i] = stage_out ? set.out[i] : nullptr;
-                }
-                if(want_work)
-                    work = set.work;
-            }
-            // half precision: a first (last) pass that converts on load (store) takes the user's
-            // array itself, and the copy on that side is not made
+            stage_in  = ep.inplace || half_io || info->load_cb;
+            stage_out = ep.inplace || half_io || info->store_cb;
+            copy_in   = stage_in;
+            copy_out  = stage_out;
+            // half precision: which sides the kernels convert themselves, and which scratch arrays
+            // the pass list then still touches.  (The scratch arrays and an allocated work area are
+            // aligned allocations: only a caller's work buffer can send the choice to the other
+            // pass list, which has no converting kernels.)
             if(half_io && !g_no_half_fuse)
             {
-                void* s_in[2]  = {st_in[0], st_in[1]};
-                void* s_out[2] = {st_out[0], st_out[1]};
-                if(&select_exec_plan(ep, s_in, s_out, work) == &ep)
+                void* const aligned_stub   = reinterpret_cast<void*>(uintptr_t(4096));
+                void*       probe[2]       = {aligned_stub, aligned_stub};
+                const void* const probe_wk = work ? work : aligned_stub;
+                if(&select_exec_plan(ep, probe, probe, probe_wk) == &ep)
                 {
                     ehalf.in       = in[0];
                     ehalf.out      = out[0];
                     ehalf.fuse_in  = !in_planar && half_fusable(ep, true, in[0]);
                     ehalf.fuse_out = !out_planar && half_fusable(ep, false, out[0]);
+                    half_scratch_needs(ep, ehalf.fuse_in, ehalf.fuse_out, stage_in, stage_out);
+                    copy_in  = !ehalf.fuse_in;
+                    copy_out = !ehalf.fuse_out;
+                    if(ep.inplace)
+                        stage_in = stage_out = stage_in || stage_out;
                 }
             }
+            const size_t want_work = (need && !work) ? need : 0;
+            if(stage_in || stage_out || want_work)
+            {
+                stage_guard.lock();
+                StageSet&  set  = plan->stage[stream];
+                const bool fits = (!stage_in || (set.in[0].bytes >= in_bytes && (nin < 2 || set.in[1].bytes >= in_bytes)))
+                                  && (!stage_out || ep.inplace
+                                      || (set.out[0].bytes >= out_bytes && (nout < 2 || set.out[1].bytes >= out_bytes)))
+                                  && set.work.bytes >= want_work;
+                if(!fits)
+                {
+                    // allocating: not in the variant that may not, and not while the stream is
+                    // being captured
+                    if(static_work || fftrt_stream_capturing(stream))
+                        return rocfft_status_failure;
+                    bool ok = true;
+                    for(int i = 0; i < nin && ok && stage_in; ++i)
+                        ok = plan->stage_grow(set.in[i], in_bytes);
+                    for(int i = 0; i < nout && ok && stage_out && !ep.inplace; ++i)
+                        ok = plan->stage_grow(set.out[i], out_bytes);
+                    if(ok && want_work)
+                        ok = plan->stage_grow(set.work, want_work);
+                    if(!ok)
+                        return rocfft_status_failure;
+                }
+                for(int i = 0; i < 2; ++i)
+                {
+                    st_in[i]  = stage_in ? set.in[i].ptr : nullptr;
+                    st_out[i] = stage_out ? (ep.inplace ? set.in[i].ptr : set.out[i].ptr) : nullptr;
+                }
+                if(want_work)
+                    work = set.work.ptr;
+            }
             bool ok = true;
-            for(int i = 0; i < nin && ok && stage_in && !ehalf.fuse_in; ++i)
+            for(int i = 0; i < nin && ok && copy_in; ++i)
             {
                 cin.store   = 0;
                 cin.offset  = (int64_t)pr.ioffset[i];
@@ -684,11 +688,13 @@ static rocfft_status execute_impl(const rocfft_plan plan, void* in_buffer[], voi
             if(!ok)
                 return rocfft_status_failure;
         }
+        // (a side without scratch array that the kernels convert themselves: the pointer handed on
+        // is never used, the pass takes ehalf.in / ehalf.out)
         void* run_in[2]  = {stage_in ? st_in[0] : in[0], stage_in ? st_in[1] : in[1]};
         void* run_out[2] = {stage_out ? st_out[0] : out[0], stage_out ? st_out[1] : out[1]};
         rocfft_status st = run_exec_plan(ep, run_in, run_out, work, stream, pass_ms, fused ? &ecb : nullptr,
                                          (ehalf.fuse_in || ehalf.fuse_out) ? &ehalf : nullptr);
-        for(int i = 0; i < nout && st == rocfft_status_success && stage_out && !ehalf.fuse_out; ++i)
+        for(int i = 0; i < nout && st == rocfft_status_success && copy_out; ++i)
         {
             cout.store   = 1;
             cout.offset  = (int64_t)pr.ooffset[i];
@@ -754,6 +760,13 @@ rocfft_status rocfft_amd_execute_static(const rocfft_plan plan, void* in_buffer[
                                         rocfft_execution_info info)
 {
     return execute_impl(plan, in_buffer, out_buffer, info, nullptr, true);
+}
+
+rocfft_status rocfft_amd_copy_probe(const rocfft_amd_probe* probe, void* stream)
+{
+    if(!probe)
+        return rocfft_status_invalid_arg_value;
+    return fftrt_copy_probe(probe, stream) == 0 ? rocfft_status_success : rocfft_status_failure;
 }
 
 rocfft_status rocfft_amd_plan_get_pass_count(const rocfft_plan plan, size_t* count)

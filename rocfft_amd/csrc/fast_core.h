@@ -210,6 +210,18 @@ FFT_DEV void fk_compute_tw(const typename cplx_of<T>::type* t, uint32_t tt, type
     }
 }
 
+// Workgroup barrier that orders LDS traffic only.  The exchanges between passes communicate
+// through LDS alone, so global loads that are in flight (table entries requested ahead of their
+// use) need not complete here, as they would have to at a __syncthreads().
+__device__ __forceinline__ void fk_lds_barrier()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#endif
+}
+
 // all passes on register data; on entry r holds the inputs of pass 0, on exit
 // the outputs of the last pass (element (s,k) at fk_out_pos<last>)
 template <typename T, typename Cfg, typename A = FkRowAddr<Cfg>>
@@ -218,7 +230,7 @@ __device__ __forceinline__ void fk_passes_tw(const void* tw_all, typename cplx_o
                                              typename cplx_of<T>::type* r, bool lds_busy)
 {
     typedef typename cplx_of<T>::type C;
-#define FK_SYNC() __syncthreads()
+#define FK_SYNC() fk_lds_barrier()
     if(active)
         fk_compute0<T, Cfg>(tt, r);
     if constexpr(Cfg::NP > 1)
@@ -360,6 +372,59 @@ struct FkPairsOut
         pk[b] = v;
     }
 };
+// The same arrays accessed with the nontemporal hint: data that will not be read again before
+// the caches have turned over (the passes of transforms far larger than the last-level cache).
+template <typename T>
+struct FkPairsInNT
+{
+    typedef typename cplx_of<T>::type C;
+    typedef T                         V __attribute__((ext_vector_type(2)));
+    const C*                          p;
+    const C*                          first;
+    static FFT_DEV C ld(const C* q)
+    {
+        V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(q));
+        C r;
+        r.x = v.x;
+        r.y = v.y;
+        return r;
+    }
+    FFT_DEV C at(uint32_t off) const
+    {
+        return ld(p + off);
+    }
+    FFT_DEV C at2(uint64_t a, uint32_t b) const
+    {
+        const C* pk = p + a;
+        return ld(pk + b);
+    }
+    FFT_DEV C at_or_first(bool valid, uint32_t off) const
+    {
+        const C* pj = valid ? p + off : first;
+        return ld(pj);
+    }
+};
+template <typename T>
+struct FkPairsOutNT
+{
+    typedef typename cplx_of<T>::type C;
+    typedef T                         V __attribute__((ext_vector_type(2)));
+    C*                                p;
+    static FFT_DEV void st(C* q, C v)
+    {
+        V w = {v.x, v.y};
+        __builtin_nontemporal_store(w, reinterpret_cast<V*>(q));
+    }
+    FFT_DEV void put(uint32_t off, C v) const
+    {
+        st(p + off, v);
+    }
+    FFT_DEV void put2(uint64_t a, uint32_t b, C v) const
+    {
+        C* pk = p + a;
+        st(pk + b, v);
+    }
+};
 template <typename T>
 struct FkPlanarOut
 {
@@ -462,6 +527,70 @@ FFT_DEV uint32_t fk_w_out(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
     return (b - c.b0) * p.w2_os_c + (g - b * p.w_inner) * p.w_os_c;
 }
 
+// The large twiddles W_L^{j q} of a thread's outputs j = ot + s TPT + k CL of the last pass, in
+// factored form: W^{q ot} . W^{q s TPT} . W^{q (k mod 4) CL} . W^{q 4 (k div 4) CL} (the last two
+// as one factor when the radix is no multiple of 4).  A thread with S x R outputs looks up
+// 1 + (S-1) + 3 + (R/4-1) table values instead of S R of them -- 7 instead of 16 for 64 points
+// in 4 threads, or for one radix-16 butterfly a thread -- and every twiddle is the product of
+// at most four table values, each the product of the two entries of the two-level table.  The
+// lookups depend only on the thread's place in the tile, so a kernel can issue them before it
+// loads its data (fetch) and form the table values while the data is on its way (combine);
+// the dependent round trip to the tables then no longer sits between the last butterfly and
+// the stores.
+template <typename T, typename Cfg>
+struct FkStoreTwiddles
+{
+    typedef typename cplx_of<T>::type C;
+    static constexpr int              LAST   = Cfg::NP - 1;
+    static constexpr int              RL     = Cfg::radix(LAST);
+    static constexpr int              SL     = Cfg::S(LAST);
+    static constexpr int              CL     = Cfg::N / RL;
+    static constexpr bool             SPLITK = RL > 4 && RL % 4 == 0;
+    static constexpr int              KL     = SPLITK ? 4 : RL;
+    static constexpr int              KH     = SPLITK ? RL / 4 : 1;
+    static constexpr int              NL     = 1 + (SL - 1) + (KL - 1) + (KH - 1);
+    C                                 f[NL], g[NL];
+    FFT_DEV void fetch(const fftk_params& p, uint32_t ot, uint32_t oq)
+    {
+        const C*       tbl  = static_cast<const C*>(p.ltw);
+        const uint32_t mask = (1u << p.ltw_shift) - 1u;
+        auto           look = [&](int i, uint32_t u) __attribute__((always_inline))
+        {
+            f[i] = tbl[u & mask];
+            g[i] = tbl[(1u << p.ltw_shift) + (u >> p.ltw_shift)];
+        };
+        look(0, ot * oq);
+#pragma unroll
+        for(int s = 1; s < SL; ++s)
+            look(s, (uint32_t)(s * Cfg::TPT) * oq);
+#pragma unroll
+        for(int k = 1; k < KL; ++k)
+            look(SL - 1 + k, (uint32_t)(k * CL) * oq);
+#pragma unroll
+        for(int k = 1; k < KH; ++k)
+            look(SL + KL - 2 + k, (uint32_t)(4 * k * CL) * oq);
+    }
+    FFT_DEV void combine()
+    {
+#pragma unroll
+        for(int i = 0; i < NL; ++i)
+            f[i] = c_mul(f[i], g[i]);
+    }
+    // twiddle of output (s, k); s and k are compile-time constants once the callers' loops are unrolled
+    FFT_DEV C at(int s, int k) const
+    {
+        const int kl = SPLITK ? (k & 3) : k, kh = SPLITK ? (k >> 2) : 0;
+        C         t  = f[0];
+        if(s)
+            t = c_mul(t, f[s]);
+        if(kl)
+            t = c_mul(t, f[SL - 1 + kl]);
+        if(kh)
+            t = c_mul(t, f[SL + KL - 2 + kh]);
+        return t;
+    }
+};
+
 // Lean path: both sides are complex arrays (interleaved pairs, or planar: in_planar /
 // out_planar) whose element offsets inside a
 // tile fit 32 bits.  Every address is a wave-uniform 64-bit base plus a 32-bit per-lane
@@ -470,7 +599,9 @@ FFT_DEV uint32_t fk_w_out(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
 // Bluestein chirp on either side, convolution mode, the fused real pre/post-processing,
 // row-in/column-out passes and (odd lengths) real samples on one side with the half spectrum
 // on the other.
-template <typename T, typename Cfg, bool HALF = false>
+// EARLY_TW: the lookups of the large twiddle on the store side are issued before the data loads;
+// EARLY_CH: so are the chirp values of the store side.
+template <typename T, typename Cfg, bool HALF = false, bool EARLY_TW = false, bool EARLY_CH = false>
 __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cplx_of<T>::type* lds,
                                                const TileCtx<T>& c, uint32_t tid, uint32_t w,
                                                uint32_t tt, bool active)
@@ -505,6 +636,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     const FkPlanarIn<T>  in_planar{static_cast<const T*>(p.in0) + c.ibase, static_cast<const T*>(p.in1) + c.ibase,
                                   static_cast<const T*>(p.in0), static_cast<const T*>(p.in1)};
     const FkPairsOut<T>  out_pairs{dst};
+    const FkPairsInNT<T>  in_pairs_nt{src, reinterpret_cast<const C*>(static_cast<const T*>(p.in0))};
+    const FkPairsOutNT<T> out_pairs_nt{dst};
     // (HALF: in0 / out0 may point at half values; ibase / obase count scalars of that array)
     const FkHalfIn<T>    in_half{reinterpret_cast<const fft_half2*>(static_cast<const _Float16*>(p.in0) + c.ibase),
                               static_cast<const fft_half2*>(p.in0)};
@@ -521,6 +654,8 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         }                           \
         else if(p.in_planar)        \
             body(in_planar);        \
+        else if(p.in_nt)            \
+            body(in_pairs_nt);      \
         else                        \
             body(in_pairs);         \
     } while(0)
@@ -534,10 +669,67 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         }                           \
         else if(p.out_planar)       \
             body(out_planar);       \
+        else if(p.out_nt)           \
+            body(out_pairs_nt);     \
         else                        \
             body(out_pairs);        \
     } while(0)
 
+    // Table values of the store side that depend on the thread's place in the tile only are
+    // requested here, before the data (the store section works the place out again below).
+    FkStoreTwiddles<T, Cfg> stw;
+    C                       ch_early[EARLY_CH ? Cfg::EPT : 1];
+    if constexpr(EARLY_TW || EARLY_CH)
+    {
+        uint32_t ow0 = w, ot0 = tt;
+        if(!p.direct_out)
+        {
+            if(p.wfast)
+            {
+                ot0 = tid % (uint32_t)Cfg::TPT;
+                ow0 = tid / (uint32_t)Cfg::TPT;
+            }
+            else
+            {
+                ow0 = tid & (p.W - 1);
+                ot0 = tid >> p.wshift;
+            }
+        }
+        // (entries beyond the tile read the tables at index 0)
+        const bool     in_tile = active && (c.tile0 + ow0 < p.tile_cnt);
+        const uint32_t oq0     = p.aux_dim == 1 ? (c.tile0 + ow0) >> p.aux_shift : c.q_block;
+        if constexpr(EARLY_TW)
+        {
+            if(p.flags & FFTK_F_TWIDDLE_STORE)
+                stw.fetch(p, in_tile ? ot0 : 0u, in_tile ? oq0 : 0u);
+        }
+        if constexpr(EARLY_CH)
+        {
+            if(p.flags & FFTK_F_CHIRP_STORE)
+            {
+                const C* chirp = static_cast<const C*>(p.chirp);
+#pragma unroll
+                for(int s = 0; s < SL; ++s)
+#pragma unroll
+                    for(int k = 0; k < RL; ++k)
+                    {
+                        const uint32_t j    = ot0 + s * Cfg::TPT + k * CL;
+                        const uint32_t idx  = j * p.chirp_js + oq0 * p.chirp_qs;
+                        const bool     keep = in_tile && idx < p.blu_n && j < p.n_out && fk_live<Cfg, LAST>(ot0, s);
+#if defined(__HIP_DEVICE_COMPILE__)
+                        const bool any_kept = __builtin_amdgcn_ballot_w64(keep) != 0;
+#else
+                        const bool any_kept = keep;
+#endif
+                        C cv;
+                        cv.x = cv.y = 0;
+                        if(any_kept)
+                            cv = chirp[keep ? idx : 0u];
+                        ch_early[s * RL + k] = cv;
+                    }
+            }
+        }
+    }
     // ---------------------------------------------------------------- load
     if(p.load_op == FFTK_LOAD_C2R_PRE)
     {
@@ -589,7 +781,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
 #pragma unroll
                 for(int i = 0; i < BINS_IT; ++i)
                     lds[tid + i * p.nthreads] = cp[i];
-                __syncthreads();
+                fk_lds_barrier();
                 if(ok)
                 {
                     const uint32_t row = w * (uint32_t)(N + 1);
@@ -605,7 +797,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     if(N % 2 == 0 && tt == 0)
                         gm = lds[row + N / 2];
                 }
-                __syncthreads();
+                fk_lds_barrier();
             }
         }
         auto fetch_pairs = [&](auto in) __attribute__((always_inline))
@@ -660,7 +852,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                 lds[fk_addr<Cfg>(w, N / 2)] = c_swap(z);
             }
         }
-        __syncthreads();
+        fk_lds_barrier();
         if(active)
             fk_read<T, Cfg, 0>(lds, w, tt, r);
         lds_busy = true;
@@ -745,7 +937,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             const uint32_t j_ = e - w_ * (uint32_t)N;
             lds[fk_addr<Cfg>(w_, j_)] = inv ? c_swap(cp[i]) : cp[i];
         }
-        __syncthreads();
+        fk_lds_barrier();
         if(active)
             fk_read<T, Cfg, 0>(lds, w, tt, r);
         lds_busy = true;
@@ -779,7 +971,20 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                             // Hermitian input of an odd-length real inverse transform (chirp index =
                             // sample index there): bins above n_in/2 are the conjugate mirror
                             const uint32_t jm = (herm && j > p.n_in / 2) ? p.n_in - j : j;
-                            C              v  = in.at_or_first(valid, jm * p.t_is_c + win);
+                            // (a slot that is padding for every lane of the wave loads nothing: half
+                            // of a power-of-two convolution length is padding)
+#if defined(__HIP_DEVICE_COMPILE__)
+                            const bool any_valid = __builtin_amdgcn_ballot_w64(valid) != 0;
+#else
+                            const bool any_valid = valid;
+#endif
+                            C v, cv;
+                            v.x = v.y = cv.x = cv.y = 0;
+                            if(any_valid)
+                            {
+                                v  = in.at_or_first(valid, jm * p.t_is_c + win);
+                                cv = chirp[valid ? idx : 0u];
+                            }
                             if(herm)
                             {
                                 if(jm != j)
@@ -788,7 +993,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                                     v.y = 0;
                             }
                             r[s * R0 + k]  = v;
-                            ch[s * R0 + k] = chirp[valid ? idx : 0u];
+                            ch[s * R0 + k] = cv;
                         }
                 };
                 if(p.load_op == FFTK_LOAD_REAL)
@@ -834,6 +1039,11 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         }
     }
 
+    if constexpr(EARLY_TW)
+    {
+        if(p.flags & FFTK_F_TWIDDLE_STORE)
+            stw.combine();
+    }
     // ---------------------------------------------------------------- transform(s)
     fk_passes<T, Cfg>(p, lds, w, tt, active, r, lds_busy);
     bool out_inv = inv;
@@ -874,7 +1084,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         else
         {
             if(Cfg::NP > 1 || lds_busy)
-                __syncthreads();
+                fk_lds_barrier();
             if(active)
             {
                 C sp[SL * RL];
@@ -897,7 +1107,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         lds[fk_addr<Cfg>(w, j)] = c_swap(c_mul(r[s * RL + k], sp[s * RL + k]));
                     }
             }
-            __syncthreads();
+            fk_lds_barrier();
             if(active)
                 fk_read<T, Cfg, 0>(lds, w, tt, r);
             fk_passes<T, Cfg>(p, lds, w, tt, active, r, true);
@@ -912,10 +1122,10 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         // half-length spectrum -> N+1 Hermitian bins (real2complex_device.h:25-103): natural
         // order through LDS, then a thread produces the pairs (j, N-j)
         if(Cfg::NP > 1 || lds_busy)
-            __syncthreads();
+            fk_lds_barrier();
         if(active)
             fk_write<T, Cfg, LAST>(lds, w, tt, r);
-        __syncthreads();
+        fk_lds_barrier();
         if constexpr(STAGE_OK)
         {
             if(p.stage_io)
@@ -940,7 +1150,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                     if(N % 2 == 0 && tt == 0)
                         zm = lds[fk_addr<Cfg>(w, N / 2)];
                 }
-                __syncthreads();
+                fk_lds_barrier();
                 if(ok)
                 {
                     const uint32_t row = w * (uint32_t)(N + 1);
@@ -986,7 +1196,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
                         lds[row + N / 2] = o;
                     }
                 }
-                __syncthreads();
+                fk_lds_barrier();
                 const uint32_t total = p.W * (uint32_t)(N + 1);
                 auto copy_out = [&](auto out) __attribute__((always_inline))
                 {
@@ -1072,10 +1282,10 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
     if(STAGE_OK && p.stage_io)
     {
         if(Cfg::NP > 1 || lds_busy)
-            __syncthreads();
+            fk_lds_barrier();
         if(active)
             fk_write<T, Cfg, LAST>(lds, w, tt, r);
-        __syncthreads();
+        fk_lds_barrier();
         const uint32_t total = p.W * N;
         const T        sc    = (p.flags & FFTK_F_SCALE) ? (T)p.scale : (T)1;
 #pragma unroll
@@ -1107,10 +1317,10 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         // order, then re-read with the lanes running along the tile dimension (or along the
         // transform) so that the global stores coalesce
         if(Cfg::NP > 1 || lds_busy)
-            __syncthreads();
+            fk_lds_barrier();
         if(active)
             fk_write<T, Cfg, LAST>(lds, w, tt, r);
-        __syncthreads();
+        fk_lds_barrier();
         if(p.wfast)
         {
             ot = tid % (uint32_t)Cfg::TPT;
@@ -1144,12 +1354,17 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         }
         if(p.flags & FFTK_F_TWIDDLE_STORE)
         {
+            if constexpr(!EARLY_TW)
+            {
+                stw.fetch(p, ot, oq);
+                stw.combine();
+            }
 #pragma unroll
             for(int s = 0; s < SL; ++s)
 #pragma unroll
                 for(int k = 0; k < RL; ++k)
                 {
-                    C tv          = large_twiddle<T>(p, (ot + s * Cfg::TPT + k * CL) * oq);
+                    const C tv    = stw.at(s, k);
                     r[s * RL + k] = out_inv ? c_mulc(r[s * RL + k], tv) : c_mul(r[s * RL + k], tv);
                 }
         }
@@ -1167,14 +1382,31 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             const C*   chirp = static_cast<const C*>(p.chirp);
             const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
             C          ch[Cfg::EPT];
+            if constexpr(EARLY_CH)
+            {
+#pragma unroll
+                for(int i = 0; i < Cfg::EPT; ++i)
+                    ch[i] = ch_early[i];
+            }
+            else
 #pragma unroll
             for(int s = 0; s < SL; ++s)
 #pragma unroll
                 for(int k = 0; k < RL; ++k)
                 {
-                    const uint32_t j   = ot + s * Cfg::TPT + k * CL;
-                    const uint32_t idx = j * p.chirp_js + oq * p.chirp_qs;
-                    ch[s * RL + k]     = chirp[(idx < p.blu_n && fk_live<Cfg, LAST>(ot, s)) ? idx : 0u];
+                    const uint32_t j    = ot + s * Cfg::TPT + k * CL;
+                    const uint32_t idx  = j * p.chirp_js + oq * p.chirp_qs;
+                    const bool     keep = idx < p.blu_n && j < p.n_out && fk_live<Cfg, LAST>(ot, s);
+#if defined(__HIP_DEVICE_COMPILE__)
+                    const bool any_kept = __builtin_amdgcn_ballot_w64(keep) != 0;
+#else
+                    const bool any_kept = keep;
+#endif
+                    C cv;
+                    cv.x = cv.y = 0;
+                    if(any_kept)
+                        cv = chirp[keep ? idx : 0u];
+                    ch[s * RL + k] = cv;
                 }
             auto emit = [&](auto out) __attribute__((always_inline))
             {
@@ -1230,7 +1462,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
 #undef FK_WITH_OUT
 }
 
-template <typename T, typename Cfg, bool VEC, bool LEAN, bool HALF = false>
+template <typename T, typename Cfg, bool VEC, bool LEAN, bool HALF = false, bool EARLY_TW = false, bool EARLY_CH = false>
 __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cplx_of<T>::type* lds)
 {
     typedef typename cplx_of<T>::type C;
@@ -1256,7 +1488,7 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
     }
     if constexpr(LEAN)
     {
-        fast_tile_lean<T, Cfg, HALF>(p, lds, c, tid, w, tt, active);
+        fast_tile_lean<T, Cfg, HALF, EARLY_TW, EARLY_CH>(p, lds, c, tid, w, tt, active);
         return;
     }
     C    r[Cfg::EPT];

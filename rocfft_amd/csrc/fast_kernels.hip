@@ -27,9 +27,10 @@ namespace
 // scale factor); 4: interleaved arrays, a scale factor, the large twiddle on the store side, the
 // fused real pre/post-processing, the tile copy of short transforms, and (single precision)
 // arrays of IEEE half pairs on the load or the store side: the first and last pass of a
-// half-precision plan, which computes in single precision.  The variants 3 and 4 are the lean
-// kernel compiled under assumptions on its arguments (fast_assume_plain): the compiler drops
-// every other path, which leaves a fifth to a third of the code and 10-50 registers fewer.
+// half-precision plan, which computes in single precision; 7, 9 and 8: the first, middle and last
+// pass of a chirp-z transform in three kernels (powers of two only).  The variants 3, 4, 7, 8, 9 are
+// the lean kernel compiled under assumptions on its arguments (fast_assume_plain): the compiler
+// drops every other path, which leaves a fifth to a third of the code and 10-50 registers fewer.
 // Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
 // their tile rows wide); no kernel here needs more than the 256 registers that leaves a thread.
 // The longest lengths need up to 1024 threads for one transform (128 registers a thread).
@@ -52,6 +53,59 @@ __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
         __builtin_assume(p.out_planar == 0);
         __builtin_assume(p.w_inner == 0);
     }
+    else if constexpr(MODE == 7)
+    {
+        // first pass of a chirp-z transform in three kernels: chirp and zero padding on the load
+        // side, the large twiddle on the store side, interleaved arrays
+        __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
+        __builtin_assume(p.store_op == FFTK_STORE_COMPLEX);
+        __builtin_assume((p.flags & ~(uint32_t)(FFTK_F_CHIRP_LOAD | FFTK_F_TWIDDLE_STORE | FFTK_F_CHIRP_CONJ)) == 0);
+        __builtin_assume((p.flags & FFTK_F_CHIRP_LOAD) != 0);
+        __builtin_assume(p.in_planar == 0);
+        __builtin_assume(p.out_planar == 0);
+        __builtin_assume(p.stage_io == 0);
+        __builtin_assume(p.w_inner == 0);
+        __builtin_assume(p.in_nt == 0);
+        __builtin_assume(p.out_nt == 0);
+    }
+    else if constexpr(MODE == 8)
+    {
+        // last pass of such a transform: chirp and scale factor on the store side
+        __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
+        __builtin_assume(p.store_op == FFTK_STORE_COMPLEX);
+        __builtin_assume((p.flags & ~(uint32_t)(FFTK_F_CHIRP_STORE | FFTK_F_SCALE | FFTK_F_CHIRP_CONJ)) == 0);
+        __builtin_assume((p.flags & FFTK_F_CHIRP_STORE) != 0);
+        __builtin_assume(p.in_planar == 0);
+        __builtin_assume(p.out_planar == 0);
+        __builtin_assume(p.stage_io == 0);
+        __builtin_assume(p.w_inner == 0);
+        __builtin_assume(p.n_in == (uint32_t)Cfg::N);
+        __builtin_assume(p.in_nt == 0);
+        __builtin_assume(p.out_nt == 0);
+    }
+    else if constexpr(MODE == 9)
+    {
+        // middle pass of such a transform: forward transform, product with the chirp spectrum,
+        // inverse transform, the large twiddle on the store side
+        __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
+        __builtin_assume(p.store_op == FFTK_STORE_COMPLEX);
+        __builtin_assume((p.flags & ~(uint32_t)(FFTK_F_CONV | FFTK_F_TWIDDLE_STORE)) == 0);
+        __builtin_assume((p.flags & FFTK_F_CONV) != 0);
+        __builtin_assume(p.in_planar == 0);
+        __builtin_assume(p.out_planar == 0);
+        __builtin_assume(p.stage_io == 0);
+        __builtin_assume(p.w_inner == 0);
+        __builtin_assume(p.n_in == (uint32_t)Cfg::N);
+        __builtin_assume(p.n_out == (uint32_t)Cfg::N);
+        __builtin_assume(p.in_nt == 0);
+        __builtin_assume(p.out_nt == 0);
+    }
+    else if constexpr(MODE == 2)
+    {
+        // (the nontemporal accesses exist in the variants for plain and twiddled passes only)
+        __builtin_assume(p.in_nt == 0);
+        __builtin_assume(p.out_nt == 0);
+    }
     else if constexpr(MODE == 3)
     {
         __builtin_assume(p.load_op == FFTK_LOAD_COMPLEX);
@@ -68,13 +122,24 @@ __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
     }
 }
 
+// Which variants request the table values of the store side (large twiddle, chirp) before
+// their data: those with registers to spare for them.  Double-precision kernels hold 64 registers
+// of data and 60 of pass twiddles; the 7 table values of the large twiddle (28 registers) fit
+// into the first pass of a chirp-z transform up to 512 points, beyond that and for the 16 chirp
+// values of the last pass the kernels spill.
+template <typename T, typename Cfg, int MODE>
+constexpr bool fast_early_twiddles()
+{
+    return MODE == 4 || ((MODE == 7 || MODE == 9) && (sizeof(T) == 4 || (MODE == 7 && Cfg::N <= 512)));
+}
+
 template <typename T, typename Cfg, int MODE>
 __global__ __launch_bounds__(fast_block_limit<Cfg>()) void fast_tile_kernel(const fftk_params p)
 {
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
     fast_assume_plain<Cfg, MODE>(p);
-    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4, fast_early_twiddles<T, Cfg, MODE>(), MODE == 8 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // The same kernel held to the registers that let WAVES waves share a SIMD.
@@ -84,7 +149,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
     fast_assume_plain<Cfg, MODE>(p);
-    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4, fast_early_twiddles<T, Cfg, MODE>(), MODE == 8 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // Waves per SIMD a kernel is compiled for; 0 = whatever its natural register count gives.
@@ -97,7 +162,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
 template <typename T, typename Cfg, int MODE>
 constexpr int fast_waves()
 {
-    return (sizeof(T) == 4 && MODE >= 3 && Cfg::TPT <= 512) ? 4 : 0;
+    return (sizeof(T) == 4 && (MODE == 3 || MODE == 4) && Cfg::TPT <= 512) ? 4 : 0;
 }
 
 template <typename T, typename Cfg, int MODE>
@@ -147,18 +212,25 @@ constexpr FastEntry fast_entry()
                          fast_variant<T, Cfg, 1, ALL_MODES != 0>(),
                          fast_variant<T, Cfg, 0, ALL_MODES != 0>(),
                          &launch_fast<T, Cfg, 3>,
-                         fast_variant<T, Cfg, 4, more>()};
+                         fast_variant<T, Cfg, 4, more>(),
+                         fast_variant<T, Cfg, 7, ALL_MODES != 0>(),
+                         fast_variant<T, Cfg, 8, ALL_MODES != 0>(),
+                         fast_variant<T, Cfg, 9, ALL_MODES != 0>()};
     }
     else
-        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr};
+        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 }
 
 #define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD, DBL)                  \
     fast_entry<SLICE, float, 0, FULL, true, FastCfg<N, A, B, C, D, TTF>>(),     \
         fast_entry<SLICE, double, 1, FULL, (DBL) != 0, FastCfg<N, A, B, C, D, (DBL) ? TTD : TTF>>(),
 
+// (a build for experiments may name a shorter list: -DFAST_SCHEDULES_FILE='"..."')
+#ifndef FAST_SCHEDULES_FILE
+#define FAST_SCHEDULES_FILE "fast_schedules.h"
+#endif
 const FastEntry g_slice[] = {
-#include "fast_schedules.h"
+#include FAST_SCHEDULES_FILE
 };
 static_assert(FAST_SLICE >= 0 && FAST_SLICE < FAST_SLICES, "compile with -DFAST_SLICE=0..FAST_SLICES-1");
 
@@ -292,8 +364,31 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
                 && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST))
             fn = e->more;
     }
+    // the first and last pass of a chirp-z transform in three kernels (kernels of their own, so
+    // that a profile tells them apart)
+    if(variants && p->lean && !p->in_planar && !p->out_planar && !p->w_inner && !p->stage_io
+       && p->load_op == FFTK_LOAD_COMPLEX && p->store_op == FFTK_STORE_COMPLEX)
+    {
+        if(e->chirp_in && (p->flags & FFTK_F_CHIRP_LOAD)
+           && (p->flags & ~(uint32_t)(FFTK_F_CHIRP_LOAD | FFTK_F_TWIDDLE_STORE | FFTK_F_CHIRP_CONJ)) == 0)
+            fn = e->chirp_in;
+        else if(e->chirp_out && (p->flags & FFTK_F_CHIRP_STORE) && p->n_in == p->n
+                && (p->flags & ~(uint32_t)(FFTK_F_CHIRP_STORE | FFTK_F_SCALE | FFTK_F_CHIRP_CONJ)) == 0)
+            fn = e->chirp_out;
+        else if(e->chirp_mid && (p->flags & FFTK_F_CONV) && p->n_in == p->n && p->n_out == p->n
+                && (p->flags & ~(uint32_t)(FFTK_F_CONV | FFTK_F_TWIDDLE_STORE)) == 0)
+            fn = e->chirp_mid;
+    }
     if(!fn)
         return FFTRT_NO_FAST_VARIANT;
+    fftk_params without_nt;
+    if((p->in_nt || p->out_nt) && fn != e->plain && fn != e->more)
+    {
+        without_nt        = *p;
+        without_nt.in_nt  = 0;
+        without_nt.out_nt = 0;
+        p                 = &without_nt;
+    }
     return fn(p, grid, lds_bytes, stream);
 }
 #endif

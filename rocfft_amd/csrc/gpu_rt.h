@@ -76,6 +76,10 @@ int fftrt_launch_big32k(const struct fftk_big_params* p, void* stream);
 #define FFTRT_STATIC_SCRATCH_BYTES (64u << 20)
 int fftrt_static_scratch(void** ptr, size_t* bytes);
 
+// plain copies in the access shapes of the passes (rocfft_amd.h: rocfft_amd_copy_probe)
+struct rocfft_amd_probe;
+int fftrt_copy_probe(const struct rocfft_amd_probe* q, void* stream);
+
 // event timing, used by the optional per-pass profile log
 int fftrt_event_create(void** ev);
 int fftrt_event_destroy(void* ev);

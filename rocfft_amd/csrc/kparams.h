@@ -93,6 +93,7 @@ struct fftk_params
     uint32_t t_is_c, t_os_c, w_is_c, w_os_c;
     uint32_t in_planar, out_planar; // lean path: that side is a planar complex array (real parts
                                     // at in0/out0, imaginary parts at in1/out1)
+    uint32_t in_nt, out_nt;     // lean path, interleaved arrays: access that side with the nontemporal hint
     uint32_t in_half, out_half; // lean path, single precision: that side is an array of IEEE half
                                 // pairs (in0 / out0 point at half values, strides and offsets count
                                 // half scalars)

@@ -11,6 +11,7 @@
 #include <mutex>
 #include <sstream>
 #include <stdexcept>
+#include <thread>
 
 namespace fftamd
 {
@@ -111,6 +112,29 @@ struct HostTable
         v.push_back(s);
     }
 };
+
+// fn(first, last) over [0, n) on the host's threads (long tables: the chirp of a prime length in
+// the millions costs seconds on one thread)
+template <typename Fn>
+static void host_parallel(uint64_t n, Fn fn)
+{
+    unsigned workers = std::min<unsigned>(16, std::max(1u, std::thread::hardware_concurrency()));
+    if(n < (1u << 16) || workers < 2)
+    {
+        fn((uint64_t)0, n);
+        return;
+    }
+    std::vector<std::thread> pool;
+    const uint64_t           step = (n + workers - 1) / workers;
+    for(unsigned w = 0; w < workers; ++w)
+    {
+        const uint64_t a = std::min<uint64_t>(n, w * step), b = std::min<uint64_t>(n, a + step);
+        if(a < b)
+            pool.emplace_back([=]() { fn(a, b); });
+    }
+    for(std::thread& t : pool)
+        t.join();
+}
 
 static std::mutex                                   g_cache_mutex;
 static std::map<std::string, std::weak_ptr<DeviceTable>> g_cache;
@@ -275,12 +299,11 @@ static TablePtr chirp_table(uint64_t N, int precision, bool dry)
     std::ostringstream key;
     key << "chirp_" << N;
     return cached_table(key.str(), precision, dry, [&](HostTable& h) {
-        for(uint64_t m = 0; m < N; ++m)
-        {
-            long double c, s;
-            chirp_value(m, N, c, s);
-            h.push(c, s);
-        }
+        h.v.resize(2 * N);
+        host_parallel(N, [&](uint64_t first, uint64_t last) {
+            for(uint64_t m = first; m < last; ++m)
+                chirp_value(m, N, h.v[2 * m], h.v[2 * m + 1]);
+        });
     });
 }
 
@@ -1231,6 +1254,38 @@ static void split_three(uint64_t n, size_t esize, bool column, uint64_t& n2, uin
     }
 }
 
+// n = n3 * n2 * n1 * n0 for the four-pass scheme: one more strided factor outside split_three
+static void split_four(uint64_t n, size_t esize, bool column, uint64_t& n3, uint64_t& n2, uint64_t& n1,
+                       uint64_t& n0)
+{
+    n3 = n2 = n1 = n0 = 0;
+    double best_score = -1;
+    for(uint64_t a = 2; a < n; ++a)
+    {
+        if(n % a || !column_kernel_length(a, esize))
+            continue;
+        uint64_t b2, b1, b0;
+        split_three(n / a, esize, column, b2, b1, b0);
+        if(b2 == 0)
+            continue;
+        double score = (fast_kernel_exists(a, esize) ? 2.0 : 0.0) + (fast_kernel_exists(b2, esize) ? 2.0 : 0.0)
+                       + (fast_kernel_exists(b1, esize) ? 2.0 : 0.0) + (fast_kernel_exists(b0, esize) ? 2.0 : 0.0);
+        // similar strided factors, the long one in the row pass
+        const uint64_t lo = std::min(a, std::min(b2, b1)), hi = std::max(a, std::max(b2, b1));
+        score += (double)lo / (double)hi + (double)b0 / (double)n;
+        if(a < 8)
+            score -= 1.0;
+        if(score > best_score)
+        {
+            best_score = score;
+            n3         = a;
+            n2         = b2;
+            n1         = b1;
+            n0         = b0;
+        }
+    }
+}
+
 static bool smooth(uint64_t n)
 {
     std::vector<uint32_t> r;
@@ -1350,68 +1405,94 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
             fail("this real-transform length needs a decomposition that is not implemented");
         // The row pass of the two-pass scheme stores transposed, W rows at a time; beyond 512
         // points per row W gets too small for coalesced stores, and three passes are faster.
-        uint64_t n1, n0, n2 = 0;
-        split_two(n, esize, column, n1, n0, 512);
+        // (ROCFFT_AMD_SPLIT_LEVELS=3 or 4 asks for that many passes where fewer would do: tests)
+        const char* want_env = getenv("ROCFFT_AMD_SPLIT_LEVELS");
+        const int   want     = want_env ? atoi(want_env) : 0;
+        uint64_t n1 = 0, n0 = 0, n2 = 0;
+        if(want < 3)
+            split_two(n, esize, column, n1, n0, 512);
         if(n1 == 0)
         {
-            split_three(n, esize, column, n2, n1, n0);
-            if(n2 == 0)
+            if(want < 4)
+                split_three(n, esize, column, n2, n1, n0);
+            if(n2 == 0 && want < 3)
                 split_two(n, esize, column, n1, n0);
+            if(n2 == 0)
+                n1 = want >= 3 ? 0 : n1;
         }
+        std::vector<uint64_t> levels; // strided factors from the outermost in, then the row factor
         if(n2 != 0)
+            levels = {n2, n1, n0};
+        else if(n1 == 0)
         {
-            // Three passes, n = n2 * (n1 * n0): a column FFT over the n2 samples that are
-            // R = n1*n0 apart times W_n^{k2 r}; then each contiguous run of R points is
-            // transformed by the two-pass scheme (column FFT over n1 times W_R^{k1 n0'}, row
-            // FFT over n0), the last pass storing result k2 + n2*(k1 + n1*k0).
-            const uint64_t R = n1 * n0;
+            // four passes: one more strided factor outside the three-pass scheme
+            uint64_t a3, a2, a1, a0;
+            split_four(n, esize, column, a3, a2, a1, a0);
+            if(a3 != 0)
+                levels = {a3, a2, a1, a0};
+        }
+        if(!levels.empty())
+        {
+            // Several passes, n = f0 f1 ... fL: pass i < L is a column FFT over the f_i samples that
+            // lie R_i = f_{i+1} ... f_L apart inside each contiguous run of f_i R_i points, times
+            // W_{f_i R_i}^{k_i r} (r the position inside the run of R_i); the last pass transforms the
+            // contiguous runs of f_L points and stores result k_0 + f_0 (k_1 + f_1 (k_2 + ...)).
+            // (Pass 0 reads the user's array, the others work in place in the scratch array.)
+            const size_t L = levels.size() - 1;
+            std::vector<uint64_t> R(L + 1, 1);
+            for(size_t i = L; i-- > 0;)
+                R[i] = R[i + 1] * levels[i + 1];
             b.need_tmp(lines * n);
             std::vector<int64_t> pk = packed_strides(n);
+            for(size_t i = 0; i < L; ++i)
             {
                 TileSpec s = base_spec();
-                s.n        = (uint32_t)n2;
-                s.t_is     = (int64_t)R * t_is;
-                s.t_os     = (int64_t)R * 2;
-                s.src      = src;
+                s.n        = (uint32_t)levels[i];
+                s.t_is     = (int64_t)R[i] * (i == 0 ? t_is : 2);
+                s.t_os     = (int64_t)R[i] * 2;
+                s.src      = i == 0 ? src : tmp;
                 s.dst      = tmp;
-                s.others.push_back({(uint32_t)R, t_is, 2, true});
-                add_others(s, true, false, pk);
+                s.others.push_back({(uint32_t)R[i], i == 0 ? t_is : 2, 2, true});
+                for(size_t j = 0; j < i; ++j)
+                    s.others.push_back({(uint32_t)levels[j], (int64_t)R[j] * 2, (int64_t)R[j] * 2, false});
+                add_others(s, i == 0, false, pk);
                 s.flags |= FFTK_F_TWIDDLE_STORE;
-                s.ltw       = large_twiddles(n, b.precision, b.dry);
-                s.ltw_shift = large_twiddle_shift(n);
-                s.note      = dims_note("split3 A (column fft over the outer factor + twiddle)", n2);
+                const uint64_t span = levels[i] * R[i];
+                s.ltw               = large_twiddles(span, b.precision, b.dry);
+                s.ltw_shift         = large_twiddle_shift(span);
+                static const char* names[3] = {"A (column fft over the outer factor + twiddle)",
+                                               "B (column fft over the middle factor + twiddle)",
+                                               "B2 (column fft over the inner strided factor + twiddle)"};
+                s.note = dims_note((std::string(L == 2 ? "split3 " : "split4 ") + names[i]).c_str(), levels[i]);
                 b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
             }
             {
                 TileSpec s = base_spec();
-                s.n        = (uint32_t)n1;
-                s.t_is = s.t_os = (int64_t)n0 * 2;
-                s.src = s.dst = tmp;
-                s.others.push_back({(uint32_t)n0, 2, 2, true});
-                s.others.push_back({(uint32_t)n2, (int64_t)R * 2, (int64_t)R * 2, false});
-                add_others(s, false, false, pk);
-                s.flags |= FFTK_F_TWIDDLE_STORE;
-                s.ltw       = large_twiddles(R, b.precision, b.dry);
-                s.ltw_shift = large_twiddle_shift(R);
-                s.note      = dims_note("split3 B (column fft over the middle factor + twiddle)", n1);
-                b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
-            }
-            {
-                TileSpec s = base_spec();
-                s.n        = (uint32_t)n0;
+                s.n        = (uint32_t)levels[L];
                 s.t_is     = 2;
-                s.t_os     = (int64_t)(n1 * n2) * t_os;
-                s.src      = tmp;
-                s.dst      = dst;
-                s.others.push_back({(uint32_t)n1, (int64_t)n0 * 2, (int64_t)n2 * t_os, false});
-                s.others.push_back({(uint32_t)n2, (int64_t)R * 2, t_os, false});
+                uint64_t outer = 1; // f_0 ... f_{L-1}
+                for(size_t j = 0; j < L; ++j)
+                    outer *= levels[j];
+                s.t_os = (int64_t)outer * t_os;
+                s.src  = tmp;
+                s.dst  = dst;
+                uint64_t below = 1; // f_0 ... f_{j-1}
+                std::vector<Axis> ax;
+                for(size_t j = 0; j < L; ++j)
+                {
+                    ax.push_back({(uint32_t)levels[j], (int64_t)R[j] * 2, (int64_t)below * t_os, false});
+                    below *= levels[j];
+                }
+                for(size_t j = L; j-- > 0;)
+                    s.others.push_back(ax[j]);
                 add_others(s, false, true, pk);
                 if(ops.has_scale)
                 {
                     s.flags |= FFTK_F_SCALE;
                     s.scale = ops.scale;
                 }
-                s.note = dims_note("split3 C (row fft, doubly transposed store)", n0);
+                s.note = dims_note(L == 2 ? "split3 C (row fft, doubly transposed store)" : "split4 C (row fft, triply transposed store)",
+                                   levels[L]);
                 b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
             }
             return;
@@ -1769,20 +1850,22 @@ static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t 
     if(!b.dry)
     {
         std::vector<double> w(2 * M, 0.0);
-        for(uint64_t m = 0; m < N; ++m)
-        {
-            long double c, s;
-            chirp_value(m, N, c, s);
-            if(conj_chirp)
-                s = -s;
-            w[2 * m]     = (double)c;
-            w[2 * m + 1] = (double)s;
-            if(m)
+        host_parallel(N, [&](uint64_t first, uint64_t last) {
+            for(uint64_t m = first; m < last; ++m)
             {
-                w[2 * (M - m)]     = (double)c;
-                w[2 * (M - m) + 1] = (double)s;
+                long double c, s;
+                chirp_value(m, N, c, s);
+                if(conj_chirp)
+                    s = -s;
+                w[2 * m]     = (double)c;
+                w[2 * m + 1] = (double)s;
+                if(m)
+                {
+                    w[2 * (M - m)]     = (double)c;
+                    w[2 * (M - m) + 1] = (double)s;
+                }
             }
-        }
+        });
         void* dbuf = nullptr;
         if(fftrt_malloc(&dbuf, 2 * M * sizeof(double)) != 0)
             fail("device allocation failed");
@@ -2278,9 +2361,14 @@ static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t 
         tstride[i] = run;
         run *= (int64_t)len[i];
     }
-    const int64_t rowS = run + 64; // padded pitch between rows of dimension e
-    const int64_t s_n1 = rowS, s_n0 = (int64_t)n1 * rowS;
-    run                = (int64_t)n * rowS;
+    // Padded pitch between the rows of dimension e: 512 bytes more than a row (measured on the
+    // 4096 x 4096 single-precision transform: no padding, pass B 0.435 ms; 256 bytes, 0.488 ms --
+    // every other row then starts in the middle of a 512-byte block; 512 bytes, 0.408 ms; 1 KB,
+    // 0.416 ms; 4 KB, 0.441 ms).  ROCFFT_AMD_STAGE_PAD sets it in scalars (comparisons).
+    static const char* pad_env = getenv("ROCFFT_AMD_STAGE_PAD");
+    const int64_t      rowS    = run + (pad_env ? atol(pad_env) : (int64_t)(512 / (esize / 2)));
+    const int64_t      s_n1 = rowS, s_n0 = (int64_t)n1 * rowS;
+    run                = (int64_t)n0 * s_n0;
     for(size_t i = e + 1; i < rank; ++i)
     {
         tstride[i] = run;
@@ -2403,8 +2491,14 @@ static void check_sizes(const Problem& p)
         throw PlanError(rocfft_status_failure, "bad batch");
 }
 
-static rocfft_status build_exec_plan_once(const Problem& p, ExecPlan& plan, bool dry, std::string& err)
+static rocfft_status build_exec_plan_once(const Problem& given, ExecPlan& plan, bool dry, std::string& err)
 {
+    // One transform: the distances between transforms are never used, and an in-place plan may
+    // name different ones for its two sides (the reference's tests do: clients/tests/
+    // accuracy_test_adhoc.cpp:84-157).
+    Problem p = given;
+    if(p.batch == 1)
+        p.idist = p.odist = 0;
     try
     {
         if(p.precision != rocfft_precision_single && p.precision != rocfft_precision_double)
@@ -2831,6 +2925,54 @@ bool half_fusable(const ExecPlan& plan, bool input, const void* user)
     return ((uintptr_t)(static_cast<const char*>(user) + io.off0 * 2) % 4) == 0;
 }
 
+void half_scratch_needs(const ExecPlan& plan, bool fuse_in, bool fuse_out, bool& need_in, bool& need_out)
+{
+    need_in = need_out = false;
+    const size_t n = plan.passes.size();
+    for(size_t i = 0; i < n; ++i)
+    {
+        const PassRec& r     = plan.passes[i];
+        const bool     first = i == 0, last = i + 1 == n;
+        if(r.src.buf == BUF_IN && !(first && fuse_in))
+            need_in = true;
+        if(r.src.buf == BUF_OUT)
+            need_out = true;
+        // (in place the output array is the input array; out of place a real inverse transform
+        // may still work on its input array)
+        if(r.dst.buf == BUF_OUT && !(last && fuse_out))
+            need_out = true;
+        if(r.dst.buf == BUF_IN && !(plan.inplace && last && fuse_out))
+            need_in = true;
+    }
+    if(plan.inplace)
+        need_in = need_out = need_in || need_out;
+}
+
+// Single-precision passes that move far more data than the last-level cache holds (256 MB) read
+// and write interleaved arrays with the nontemporal hint: nothing they touch is used again
+// before it would be evicted anyway.  Measured on MI355X: 4096 x 4096 x 8 transform 1.31 -> 1.23 ms,
+// 65536 rows of 4096 points 0.81 -> 0.79 ms.  Only where every contiguous run of a tile on that
+// side starts and ends on a 128-byte line: on tiles that share lines with their neighbours the
+// hint keeps the halves from merging in the cache (512 x 512 x 257 double-precision columns,
+// 257 bins a row: 0.43 -> 0.84 ms), and double-precision passes measured 3-8 % slower with it.
+static const double NT_MIN_MBYTES = 768.0;
+static bool pass_streams_side(const fftk_params& k, bool in)
+{
+    const int64_t line = 32; // scalars of 4 bytes per 128-byte line
+    if((in ? k.in_planar : k.out_planar) || k.w_inner)
+        return false;
+    const int64_t  t = in ? k.t_is : k.t_os, w = in ? k.w_is : k.w_os;
+    const bool     fast_tile = in ? k.in_fast_tile != 0 : k.out_fast_tile != 0;
+    const int64_t* o = in ? k.o_is : k.o_os;
+    for(int i = 0; i < 3; ++i)
+        if(k.oc[i] > 1 && o[i] % line)
+            return false;
+    if(fast_tile) // runs of W elements along the tile axis
+        return w == 2 && (k.W * 2) % line == 0 && t % line == 0 && k.tile_cnt % k.W == 0;
+    // runs of n elements along the transform
+    return t == 2 && ((int64_t)k.n * 2) % line == 0 && (k.tile_cnt == 1 || w % line == 0);
+}
+
 rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const out[2], void* work,
                             void* stream, float* pass_ms, const ExecCallbacks* cb, const ExecHalf* half)
 {
@@ -3032,6 +3174,17 @@ rocfft_status run_exec_plan(const ExecPlan& plan, void* const in[2], void* const
                    || (!k.out_half && !aligned(k.out0, plan.elem_bytes)))
                     return rocfft_status_failure;
                 k.lean = 1;
+            }
+            // Nontemporal accesses (see pass_streams_side): ROCFFT_AMD_NO_NT=1 switches them off,
+            // ROCFFT_AMD_NT_MB sets the least data volume of a pass in megabytes (comparisons)
+            {
+                static const bool   nt_on  = !getenv("ROCFFT_AMD_NO_NT");
+                static const double nt_min = (getenv("ROCFFT_AMD_NT_MB") ? atof(getenv("ROCFFT_AMD_NT_MB")) : NT_MIN_MBYTES) * 1e6;
+                if(nt_on && k.lean && plan.precision == 0 && rec.bytes_rw >= nt_min && !with_cb)
+                {
+                    k.in_nt  = pass_streams_side(k, true) && !k.in_half && aligned(k.in0, 128) ? 1 : 0;
+                    k.out_nt = pass_streams_side(k, false) && !k.out_half && aligned(k.out0, 128) ? 1 : 0;
+                }
             }
             rc = fftrt_launch_tile(&k, plan.precision, vec ? 1 : 0, rec.grid, rec.lds, stream);
         }

@@ -147,6 +147,10 @@ struct ExecHalf
 };
 // can the first (input = true) / last pass of the list take the user's half array at `user`?
 bool half_fusable(const ExecPlan& plan, bool input, const void* user);
+// Which single-precision scratch arrays (standing in for the user's input and output arrays) the
+// pass list still touches when its first pass reads (fuse_in) / its last pass writes (fuse_out)
+// the user's half array itself.  In place there is one array: both answers are the same.
+void half_scratch_needs(const ExecPlan& plan, bool fuse_in, bool fuse_out, bool& need_in, bool& need_out);
 
 // Enqueues every pass on `stream`.  in/out hold one pointer (interleaved, real)
 // or two (planar).  `work` must hold plan.work_bytes() bytes when that is non-zero.

@@ -298,6 +298,10 @@ int fftrt_static_scratch(void** ptr, size_t* bytes)
     *bytes = area.size();
     return 0;
 }
+int fftrt_copy_probe(const struct rocfft_amd_probe*, void*)
+{
+    return 1; // measurement only: nothing to time without a device
+}
 int fftrt_event_create(void** ev)
 {
     *ev = nullptr;

@@ -128,9 +128,10 @@ def test_callbacks_on_the_gpu(gpu_lib, which):
 @pytest.mark.gpu
 def test_callbacks_and_half_precision_replay_from_a_graph(gpu_lib):
     """Callbacks are called from inside the first and last kernel of the plan: an execution
-    with callbacks allocates nothing and can be captured into a graph straight away.  Half
-    precision stages through copies in buffers the plan owns per stream: the first execution
-    on a stream allocates them (so it cannot be the captured one), later ones allocate nothing.
+    with callbacks allocates nothing and can be captured into a graph straight away, and so can
+    a half-precision plan whose one kernel converts on load and store.  A half-precision plan of
+    several kernels keeps its single-precision intermediate array per stream: the first execution
+    on a stream allocates it (so it cannot be the captured one), later ones allocate nothing.
     Every replay is checked against an eager result, with eager work between the replays."""
     import torch
 
@@ -171,13 +172,36 @@ def test_callbacks_and_half_precision_replay_from_a_graph(gpu_lib):
             assert err < 1e-5 * (rep + 2), (n, rep, err)
         assert torch.equal(xin, x * 4), n  # out of place: the input is left alone
 
-    # half precision
+    # half precision, one kernel that reads and writes the half arrays itself: no scratch copy,
+    # the first execution can be the captured one
     hplan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256], 4, lib=lib)
     xh = (torch.rand((4, 256, 2), generator=gen, device=dev) - 0.5).to(torch.float16)
     yh = torch.zeros_like(xh)
     hinfo = B.ExecutionInfo(lib).set_stream(side.cuda_stream)
     torch.cuda.synchronize()
-    # before the plan has buffers for this stream, a captured execution is refused
+    gh = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(gh, stream=side):
+            first = hplan.execute_status([xh.data_ptr()], [yh.data_ptr()], hinfo)
+    assert first == 0
+    torch.cuda.synchronize()
+    xq = torch.view_as_complex(xh.to(torch.float32).contiguous())
+    href = torch.view_as_real(torch.fft.fft(xq, dim=1))
+    for rep in range(2):
+        yh.zero_()
+        torch.cuda.synchronize()
+        gh.replay()
+        torch.cuda.synchronize()
+        err = (torch.linalg.vector_norm(yh.to(torch.float32) - href) / torch.linalg.vector_norm(href)).item()
+        assert err < 1.5e-3, (rep, err)
+
+    # half precision with a single-precision intermediate array (two kernels): the plan keeps it
+    # per stream, the first execution on a stream allocates it (so it cannot be the captured
+    # one), later ones allocate nothing
+    hplan = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256, 256], 2, lib=lib)
+    xh = (torch.rand((2, 256 * 256, 2), generator=gen, device=dev) - 0.5).to(torch.float16)
+    yh = torch.zeros_like(xh)
+    torch.cuda.synchronize()
     g0 = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
         with torch.cuda.graph(g0, stream=side):

@@ -271,6 +271,19 @@ def test_long_1d(gpu, n):
         H.check(lib, be, B.REAL_INVERSE, [n], 2, B.DOUBLE, inplace=True)
 
 
+def test_four_pass_split(gpu, monkeypatch):
+    """one more strided pass than the longest lengths of three passes need, asked for at lengths
+    the checker finishes (the lengths that need it are run by tests/test_reference_matrix.py)"""
+    lib, be = gpu
+    monkeypatch.setenv("ROCFFT_AMD_SPLIT_LEVELS", "4")
+    for n in (65536, 2 ** 20, 3 ** 9, 5 ** 8, 30030):
+        H.check(lib, be, B.COMPLEX_FORWARD, [n], 2, B.SINGLE)
+        H.check(lib, be, B.COMPLEX_INVERSE, [n], 1, B.DOUBLE, inplace=True, scale=0.5)
+    monkeypatch.setenv("ROCFFT_AMD_SPLIT_LEVELS", "3")
+    H.check(lib, be, B.COMPLEX_FORWARD, [32768], 2, B.SINGLE)
+    H.check(lib, be, B.COMPLEX_FORWARD, [2 ** 17], 2, B.DOUBLE)
+
+
 @pytest.mark.parametrize("lengths", [[8193], [10007], [19683], [15625], [100003], [9999, 3], [3, 9999]])
 def test_long_odd_real(gpu, lengths):
     lib, be = gpu

@@ -94,8 +94,52 @@ def test_static_work_area_limit(gpu_lib):
     torch.cuda.synchronize()
     assert st == B.STATUS_INVALID_WORK_BUFFER
     assert (y == 7.0).all()
-    # half precision stages through per-call buffers: refused as well
-    half = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256], 4, lib=lib)
-    xh = torch.zeros((4, 256, 2), dtype=torch.float16, device=dev)
+    # half precision with a single-precision intermediate array, which the plan would have to
+    # allocate: refused as well
+    half = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [256, 256], 2, lib=lib)
+    xh = torch.zeros((2, 256 * 256, 2), dtype=torch.float16, device=dev)
     yh = torch.zeros_like(xh)
     assert half.execute_static_status([xh.data_ptr()], [yh.data_ptr()]) == B.STATUS_FAILURE
+
+
+def test_static_variant_allocates_no_device_memory(gpu_lib):
+    """free device memory (as the driver reports it) is the same before and after the calls;
+    half-precision and callback plans whose kernels do the conversion / call the callbacks
+    themselves are accepted"""
+    import torch
+
+    from test_callbacks import S_LOAD, S_STORE, callback_library
+
+    lib = gpu_lib
+    dev = torch.device("cuda:0")
+    big = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [1 << 17], 16, lib=lib)
+    x = _complex_input(torch, dev, 21, 16, 1 << 17, torch.complex64)
+    y = torch.empty_like(x)
+    half = B.Plan(B.NOTINPLACE, B.COMPLEX_FORWARD, B.HALF, [1024], 64, lib=lib)
+    xh = (torch.view_as_real(_complex_input(torch, dev, 22, 64, 1024, torch.complex64))).to(torch.float16)
+    yh = torch.zeros_like(xh)
+    cblib = callback_library("libcb_device.so")
+    scales = torch.tensor([S_LOAD, S_STORE], dtype=torch.float32, device=dev)
+    cinfo = B.ExecutionInfo(lib)
+    cinfo.set_load_callback(cblib.cb_get(0, 1, 0), scales[0:].data_ptr())
+    cinfo.set_store_callback(cblib.cb_get(1, 1, 0), scales[1:].data_ptr())
+    yc = torch.empty_like(x)
+    # one warm-up of each kernel (code objects are loaded on first use), then measure
+    big.execute_static([x.data_ptr()], [y.data_ptr()])
+    half.execute_static([xh.data_ptr()], [yh.data_ptr()])
+    big.execute_static([x.data_ptr()], [yc.data_ptr()], cinfo)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        big.execute_static([x.data_ptr()], [y.data_ptr()])
+        half.execute_static([xh.data_ptr()], [yh.data_ptr()])
+        big.execute_static([x.data_ptr()], [yc.data_ptr()], cinfo)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    ref = torch.fft.fft(x, dim=1)
+    assert (torch.linalg.vector_norm(y - ref) / torch.linalg.vector_norm(ref)).item() < 1e-5
+    assert (torch.linalg.vector_norm(yc - ref * (S_LOAD * S_STORE)) / torch.linalg.vector_norm(ref)).item() < 2e-5
+    href = torch.view_as_real(torch.fft.fft(torch.view_as_complex(xh.to(torch.float32).contiguous()), dim=1))
+    err = (torch.linalg.vector_norm(yh.to(torch.float32) - href) / torch.linalg.vector_norm(href)).item()
+    assert err < 1.5e-3, err
