@@ -117,6 +117,8 @@ typedef struct rocfft_amd_probe
     unsigned    tile_width, elem_bytes, tiles_per_slab;
     size_t      in_slab, out_slab;
     int         resident_grid; /* tiles: 1 = a resident grid strides through the tiles, 0 = one workgroup per tile */
+    int         xcd_ranges;    /* tiles, one workgroup per tile: 1 = workgroups renumbered so that each of the 8 XCDs
+                                  works through one contiguous range of tiles, as the column passes do */
 } rocfft_amd_probe;
 ROCFFT_EXPORT rocfft_status rocfft_amd_copy_probe(const rocfft_amd_probe* probe, void* stream);
 

@@ -89,11 +89,18 @@ __global__ __launch_bounds__(1024) void probe_rows(const v2f* in, v2f* out, size
 template <typename V>
 __global__ __launch_bounds__(256) void probe_tiles(const V* in, V* out, uint32_t W, size_t in_row, size_t out_row,
                                                    uint32_t tiles_per_slab, size_t in_slab, size_t out_slab,
-                                                   uint32_t total, int nt)
+                                                   uint32_t total, int nt, int xcd_ranges)
 {
     const uint32_t w = threadIdx.x % W, q = threadIdx.x / W, step = 256 / W;
-    for(uint32_t b = blockIdx.x; b < total; b += gridDim.x)
+    for(uint32_t b0 = blockIdx.x; b0 < total; b0 += gridDim.x)
     {
+        uint32_t b = b0;
+        if(xcd_ranges)
+        {
+            // workgroups are dealt round-robin to the 8 XCDs: give each XCD one contiguous range of tiles
+            const uint32_t xcd = b0 & 7u, idx = b0 >> 3, qd = total >> 3, rm = total & 7u;
+            b = xcd * qd + (xcd < rm ? xcd : rm) + idx;
+        }
         const uint32_t tile = b % tiles_per_slab, slab = b / tiles_per_slab;
         const V*       a    = in + (size_t)slab * in_slab + (size_t)tile * W + w;
         V*             o    = out + (size_t)slab * out_slab + (size_t)tile * W + w;
@@ -179,14 +186,15 @@ extern "C" int fftrt_copy_probe(const struct rocfft_amd_probe* q, void* stream)
         if(total >= (1ull << 31))
             return (int)hipErrorInvalidValue;
         const uint32_t grid = (uint32_t)std::min<uint64_t>(total, q->resident_grid ? (uint64_t)per_cu * cus : total);
+        const int      xcd  = (q->xcd_ranges && grid == total) ? 1 : 0;
         if(q->elem_bytes == 8)
             hipLaunchKernelGGL(probe_tiles<v2f>, dim3(grid), dim3(256), 0, s, static_cast<const v2f*>(q->src),
                                static_cast<v2f*>(q->dst), W, q->in_row, q->out_row, q->tiles_per_slab, q->in_slab,
-                               q->out_slab, (uint32_t)total, q->nontemporal);
+                               q->out_slab, (uint32_t)total, q->nontemporal, xcd);
         else if(q->elem_bytes == 16)
             hipLaunchKernelGGL(probe_tiles<v4f>, dim3(grid), dim3(256), 0, s, static_cast<const v4f*>(q->src),
                                static_cast<v4f*>(q->dst), W, q->in_row, q->out_row, q->tiles_per_slab, q->in_slab,
-                               q->out_slab, (uint32_t)total, q->nontemporal);
+                               q->out_slab, (uint32_t)total, q->nontemporal, xcd);
         else
             return (int)hipErrorInvalidValue;
         break;

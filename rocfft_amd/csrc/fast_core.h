@@ -599,9 +599,11 @@ struct FkStoreTwiddles
 // Bluestein chirp on either side, convolution mode, the fused real pre/post-processing,
 // row-in/column-out passes and (odd lengths) real samples on one side with the half spectrum
 // on the other.
-// EARLY_TW: the lookups of the large twiddle on the store side are issued before the data loads;
-// EARLY_CH: so are the chirp values of the store side.
-template <typename T, typename Cfg, bool HALF = false, bool EARLY_TW = false, bool EARLY_CH = false>
+// EARLY_TW: the lookups of the large twiddle on the store side are issued before the data loads.
+// (The chirp values of the store side stay where they are used: requested early they cost up to
+// 64 registers, and the last pass of a 1000003-point single-precision chirp-z transform went
+// from 0.115 to 0.149 ms on MI355X with three waves a SIMD instead of four.)
+template <typename T, typename Cfg, bool HALF = false, bool EARLY_TW = false>
 __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cplx_of<T>::type* lds,
                                                const TileCtx<T>& c, uint32_t tid, uint32_t w,
                                                uint32_t tt, bool active)
@@ -675,59 +677,32 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             body(out_pairs);        \
     } while(0)
 
-    // Table values of the store side that depend on the thread's place in the tile only are
-    // requested here, before the data (the store section works the place out again below).
+    // The table values of the large twiddle on the store side depend on the thread's place in the
+    // tile only and are requested here, before the data (the store section works the place out
+    // again below).
     FkStoreTwiddles<T, Cfg> stw;
-    C                       ch_early[EARLY_CH ? Cfg::EPT : 1];
-    if constexpr(EARLY_TW || EARLY_CH)
+    if constexpr(EARLY_TW)
     {
-        uint32_t ow0 = w, ot0 = tt;
-        if(!p.direct_out)
+        if(p.flags & FFTK_F_TWIDDLE_STORE)
         {
-            if(p.wfast)
+            uint32_t ow0 = w, ot0 = tt;
+            if(!p.direct_out)
             {
-                ot0 = tid % (uint32_t)Cfg::TPT;
-                ow0 = tid / (uint32_t)Cfg::TPT;
+                if(p.wfast)
+                {
+                    ot0 = tid % (uint32_t)Cfg::TPT;
+                    ow0 = tid / (uint32_t)Cfg::TPT;
+                }
+                else
+                {
+                    ow0 = tid & (p.W - 1);
+                    ot0 = tid >> p.wshift;
+                }
             }
-            else
-            {
-                ow0 = tid & (p.W - 1);
-                ot0 = tid >> p.wshift;
-            }
-        }
-        // (entries beyond the tile read the tables at index 0)
-        const bool     in_tile = active && (c.tile0 + ow0 < p.tile_cnt);
-        const uint32_t oq0     = p.aux_dim == 1 ? (c.tile0 + ow0) >> p.aux_shift : c.q_block;
-        if constexpr(EARLY_TW)
-        {
-            if(p.flags & FFTK_F_TWIDDLE_STORE)
-                stw.fetch(p, in_tile ? ot0 : 0u, in_tile ? oq0 : 0u);
-        }
-        if constexpr(EARLY_CH)
-        {
-            if(p.flags & FFTK_F_CHIRP_STORE)
-            {
-                const C* chirp = static_cast<const C*>(p.chirp);
-#pragma unroll
-                for(int s = 0; s < SL; ++s)
-#pragma unroll
-                    for(int k = 0; k < RL; ++k)
-                    {
-                        const uint32_t j    = ot0 + s * Cfg::TPT + k * CL;
-                        const uint32_t idx  = j * p.chirp_js + oq0 * p.chirp_qs;
-                        const bool     keep = in_tile && idx < p.blu_n && j < p.n_out && fk_live<Cfg, LAST>(ot0, s);
-#if defined(__HIP_DEVICE_COMPILE__)
-                        const bool any_kept = __builtin_amdgcn_ballot_w64(keep) != 0;
-#else
-                        const bool any_kept = keep;
-#endif
-                        C cv;
-                        cv.x = cv.y = 0;
-                        if(any_kept)
-                            cv = chirp[keep ? idx : 0u];
-                        ch_early[s * RL + k] = cv;
-                    }
-            }
+            // (entries beyond the tile read the table at index 0)
+            const bool     in_tile = active && (c.tile0 + ow0 < p.tile_cnt);
+            const uint32_t oq0     = p.aux_dim == 1 ? (c.tile0 + ow0) >> p.aux_shift : c.q_block;
+            stw.fetch(p, in_tile ? ot0 : 0u, in_tile ? oq0 : 0u);
         }
     }
     // ---------------------------------------------------------------- load
@@ -1382,13 +1357,6 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             const C*   chirp = static_cast<const C*>(p.chirp);
             const bool cj    = (p.flags & FFTK_F_CHIRP_CONJ) != 0;
             C          ch[Cfg::EPT];
-            if constexpr(EARLY_CH)
-            {
-#pragma unroll
-                for(int i = 0; i < Cfg::EPT; ++i)
-                    ch[i] = ch_early[i];
-            }
-            else
 #pragma unroll
             for(int s = 0; s < SL; ++s)
 #pragma unroll
@@ -1462,7 +1430,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
 #undef FK_WITH_OUT
 }
 
-template <typename T, typename Cfg, bool VEC, bool LEAN, bool HALF = false, bool EARLY_TW = false, bool EARLY_CH = false>
+template <typename T, typename Cfg, bool VEC, bool LEAN, bool HALF = false, bool EARLY_TW = false>
 __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cplx_of<T>::type* lds)
 {
     typedef typename cplx_of<T>::type C;
@@ -1488,7 +1456,7 @@ __device__ __forceinline__ void fast_tile_body(const fftk_params& p, typename cp
     }
     if constexpr(LEAN)
     {
-        fast_tile_lean<T, Cfg, HALF, EARLY_TW, EARLY_CH>(p, lds, c, tid, w, tt, active);
+        fast_tile_lean<T, Cfg, HALF, EARLY_TW>(p, lds, c, tid, w, tt, active);
         return;
     }
     C    r[Cfg::EPT];

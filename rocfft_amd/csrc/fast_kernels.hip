@@ -122,11 +122,10 @@ __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
     }
 }
 
-// Which variants request the table values of the store side (large twiddle, chirp) before
-// their data: those with registers to spare for them.  Double-precision kernels hold 64 registers
-// of data and 60 of pass twiddles; the 7 table values of the large twiddle (28 registers) fit
-// into the first pass of a chirp-z transform up to 512 points, beyond that and for the 16 chirp
-// values of the last pass the kernels spill.
+// Which variants request the table values of the large twiddle on the store side before their
+// data: those with registers to spare for them.  Double-precision kernels hold 64 registers of
+// data and 60 of pass twiddles; the 7 table values (28 registers) fit into the first pass of a
+// chirp-z transform up to 512 points, beyond that the kernels spill.
 template <typename T, typename Cfg, int MODE>
 constexpr bool fast_early_twiddles()
 {
@@ -139,7 +138,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>()) void fast_tile_kernel(cons
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
     fast_assume_plain<Cfg, MODE>(p);
-    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4, fast_early_twiddles<T, Cfg, MODE>(), MODE == 8 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4, fast_early_twiddles<T, Cfg, MODE>()>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // The same kernel held to the registers that let WAVES waves share a SIMD.
@@ -149,7 +148,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
     typedef typename cplx_of<T>::type C;
     extern __shared__ double2         smem_raw[];
     fast_assume_plain<Cfg, MODE>(p);
-    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4, fast_early_twiddles<T, Cfg, MODE>(), MODE == 8 && sizeof(T) == 4>(p, reinterpret_cast<C*>(smem_raw));
+    fast_tile_body<T, Cfg, MODE != 0, MODE >= 2, MODE == 4 && sizeof(T) == 4, fast_early_twiddles<T, Cfg, MODE>()>(p, reinterpret_cast<C*>(smem_raw));
 }
 
 // Waves per SIMD a kernel is compiled for; 0 = whatever its natural register count gives.
