@@ -460,13 +460,15 @@ def copy_probes():
         "tiles 4096 x 1 (contiguous rows of 32 KiB), one workgroup per tile": dict(tiles, tile_width=256, in_row=256, out_row=256, tiles_per_slab=1, rows=32768, in_slab=4096, out_slab=4096),
         "tiles 4096 x 1, nontemporal": dict(tiles, tile_width=256, in_row=256, out_row=256, tiles_per_slab=1, rows=32768, in_slab=4096, out_slab=4096, nontemporal=1),
         "tiles 4096 x 1, resident grid": dict(tiles, tile_width=256, in_row=256, out_row=256, tiles_per_slab=1, rows=32768, in_slab=4096, out_slab=4096, resident_grid=1),
-        # configuration 3, column passes: 64 columns x 64 rows; the rows of the intermediate array are
-        # 4096 + 64 elements apart (512 bytes of padding)
-        "tiles 64 x 64, rows 4160 apart (configuration 3, column passes)": dict(tiles, in_row=4160, out_row=4160, tiles_per_slab=64, rows=512, in_slab=64 * 4160, out_slab=64 * 4160),
-        "tiles 64 x 64, rows 4160 apart, nontemporal": dict(tiles, in_row=4160, out_row=4160, tiles_per_slab=64, rows=512, in_slab=64 * 4160, out_slab=64 * 4160, nontemporal=1),
-        "tiles 64 x 64, rows 4160 apart, resident grid": dict(tiles, in_row=4160, out_row=4160, tiles_per_slab=64, rows=512, in_slab=64 * 4160, out_slab=64 * 4160, resident_grid=1),
-        "tiles 64 x 64, rows 4128 apart (256 bytes of padding)": dict(tiles, in_row=4128, out_row=4128, tiles_per_slab=64, rows=512, in_slab=64 * 4128, out_slab=64 * 4128),
-        "tiles 64 x 64, rows 4096 apart (power-of-two pitch)": dict(tiles, in_row=4096, out_row=4096, tiles_per_slab=64, rows=512, in_slab=64 * 4096, out_slab=64 * 4096),
+        # configuration 3, column passes over 8 arrays of 4096 rows of 4096 elements: a tile is 64
+        # columns x 64 rows, the rows adjacent (first pass of the split) or 64 rows apart (second pass)
+        "tiles 64 x 64, adjacent rows of 4096 (configuration 3, first column pass)": dict(tiles, in_row=4096, out_row=4096, tiles_per_slab=64, rows=512, in_slab=64 * 4096, out_slab=64 * 4096),
+        "tiles 64 x 64, adjacent rows of 4096, nontemporal": dict(tiles, in_row=4096, out_row=4096, tiles_per_slab=64, rows=512, in_slab=64 * 4096, out_slab=64 * 4096, nontemporal=1),
+        "tiles 64 x 64, adjacent rows of 4096, resident grid": dict(tiles, in_row=4096, out_row=4096, tiles_per_slab=64, rows=512, in_slab=64 * 4096, out_slab=64 * 4096, resident_grid=1),
+        "tiles 64 x 64, rows 64 x 4096 apart (configuration 3, second column pass)": dict(tiles, in_row=64 * 4096, out_row=64 * 4096, tiles_per_slab=64, rows=512, in_slab=4096, out_slab=4096, slabs_inner=64, in_slab_outer=4096 * 4096, out_slab_outer=4096 * 4096),
+        "tiles 64 x 64, rows 64 x 4096 apart, nontemporal": dict(tiles, in_row=64 * 4096, out_row=64 * 4096, tiles_per_slab=64, rows=512, in_slab=4096, out_slab=4096, slabs_inner=64, in_slab_outer=4096 * 4096, out_slab_outer=4096 * 4096, nontemporal=1),
+        "tiles 64 x 64, adjacent rows 4096 + 32 apart (256 bytes of padding)": dict(tiles, in_row=4128, out_row=4128, tiles_per_slab=64, rows=512, in_slab=64 * 4128, out_slab=64 * 4128),
+        "tiles 64 x 64, adjacent rows 4096 + 64 apart (512 bytes of padding)": dict(tiles, in_row=4160, out_row=4160, tiles_per_slab=64, rows=512, in_slab=64 * 4160, out_slab=64 * 4160),
         # configuration 4, column passes: 8 columns of 16 bytes x 512 rows
         "tiles 8 x 512 of 16 B, rows 257 apart, each XCD a range of tiles (configuration 4, y columns)": dict(tiles, tile_width=8, elem_bytes=16, in_row=257, out_row=257, tiles_per_slab=32, rows=512, in_slab=257 * 512, out_slab=257 * 512, xcd_ranges=1),
         "tiles 8 x 512 of 16 B, rows 257 apart, workgroups round-robin over the XCDs": dict(tiles, tile_width=8, elem_bytes=16, in_row=257, out_row=257, tiles_per_slab=32, rows=512, in_slab=257 * 512, out_slab=257 * 512),
@@ -519,7 +521,7 @@ def copy_ceilings(torch, lib, names=None, reps=10):
 SHAPE_OF_CONFIG = {
     1: "tiles 4096 x 1 (contiguous rows of 32 KiB), one workgroup per tile",
     2: "rows 32769 apart read, rows of 32768 written (real inverse), 32/32",
-    3: "tiles 64 x 64, rows 4160 apart (configuration 3, column passes)",
+    3: "tiles 64 x 64, rows 64 x 4096 apart (configuration 3, second column pass)",
     4: "tiles 8 x 512 of 16 B, rows 131584 apart (configuration 4, z columns)",
     5: "tiles 4096 x 1 (contiguous rows of 32 KiB), one workgroup per tile",
 }

@@ -119,6 +119,9 @@ typedef struct rocfft_amd_probe
     int         resident_grid; /* tiles: 1 = a resident grid strides through the tiles, 0 = one workgroup per tile */
     int         xcd_ranges;    /* tiles, one workgroup per tile: 1 = workgroups renumbered so that each of the 8 XCDs
                                   works through one contiguous range of tiles, as the column passes do */
+    unsigned    slabs_inner;   /* tiles: not 0 = slab s starts at (s % slabs_inner) * in_slab + (s / slabs_inner) *
+                                  in_slab_outer (out likewise) instead of s * in_slab */
+    size_t      in_slab_outer, out_slab_outer;
 } rocfft_amd_probe;
 ROCFFT_EXPORT rocfft_status rocfft_amd_copy_probe(const rocfft_amd_probe* probe, void* stream);
 

@@ -103,7 +103,8 @@ class Probe(ctypes.Structure):
                 ("group", ctypes.c_uint), ("rows", ctypes.c_uint), ("in_row", ctypes.c_size_t),
                 ("out_row", ctypes.c_size_t), ("tile_width", ctypes.c_uint), ("elem_bytes", ctypes.c_uint),
                 ("tiles_per_slab", ctypes.c_uint), ("in_slab", ctypes.c_size_t), ("out_slab", ctypes.c_size_t),
-                ("resident_grid", ctypes.c_int), ("xcd_ranges", ctypes.c_int)]
+                ("resident_grid", ctypes.c_int), ("xcd_ranges", ctypes.c_int),
+                ("slabs_inner", ctypes.c_uint), ("in_slab_outer", ctypes.c_size_t), ("out_slab_outer", ctypes.c_size_t)]
 
 
 PROBE_STREAM, PROBE_READ, PROBE_WRITE, PROBE_ROWS, PROBE_TILES = range(5)

@@ -85,11 +85,14 @@ __global__ __launch_bounds__(1024) void probe_rows(const v2f* in, v2f* out, size
 // A tile pass's shape: a workgroup of 256 threads moves a tile of W x (4096 / W) elements
 // (W neighbouring elements are contiguous, the rows of the tile are in_row / out_row elements
 // apart), 16 elements per thread, all loads and then all stores; tiles are numbered along the
-// contiguous axis first (tiles_per_slab of them), then by slab (in_slab / out_slab elements apart).
+// contiguous axis first (tiles_per_slab of them), then by slab (in_slab / out_slab elements apart;
+// with slabs_inner set, in two levels: slabs_inner slabs that far apart, groups of them
+// in_outer / out_outer apart).
 template <typename V>
 __global__ __launch_bounds__(256) void probe_tiles(const V* in, V* out, uint32_t W, size_t in_row, size_t out_row,
                                                    uint32_t tiles_per_slab, size_t in_slab, size_t out_slab,
-                                                   uint32_t total, int nt, int xcd_ranges)
+                                                   uint32_t total, int nt, int xcd_ranges, uint32_t slabs_inner,
+                                                   size_t in_outer, size_t out_outer)
 {
     const uint32_t w = threadIdx.x % W, q = threadIdx.x / W, step = 256 / W;
     for(uint32_t b0 = blockIdx.x; b0 < total; b0 += gridDim.x)
@@ -102,8 +105,9 @@ __global__ __launch_bounds__(256) void probe_tiles(const V* in, V* out, uint32_t
             b = xcd * qd + (xcd < rm ? xcd : rm) + idx;
         }
         const uint32_t tile = b % tiles_per_slab, slab = b / tiles_per_slab;
-        const V*       a    = in + (size_t)slab * in_slab + (size_t)tile * W + w;
-        V*             o    = out + (size_t)slab * out_slab + (size_t)tile * W + w;
+        const uint32_t s_hi = slabs_inner ? slab / slabs_inner : 0, s_lo = slab - s_hi * slabs_inner;
+        const V*       a    = in + (size_t)s_lo * in_slab + (size_t)s_hi * in_outer + (size_t)tile * W + w;
+        V*             o    = out + (size_t)s_lo * out_slab + (size_t)s_hi * out_outer + (size_t)tile * W + w;
         V              r[16];
 #pragma unroll
         for(int k = 0; k < 16; ++k)
@@ -190,11 +194,13 @@ extern "C" int fftrt_copy_probe(const struct rocfft_amd_probe* q, void* stream)
         if(q->elem_bytes == 8)
             hipLaunchKernelGGL(probe_tiles<v2f>, dim3(grid), dim3(256), 0, s, static_cast<const v2f*>(q->src),
                                static_cast<v2f*>(q->dst), W, q->in_row, q->out_row, q->tiles_per_slab, q->in_slab,
-                               q->out_slab, (uint32_t)total, q->nontemporal, xcd);
+                               q->out_slab, (uint32_t)total, q->nontemporal, xcd, q->slabs_inner, q->in_slab_outer,
+                               q->out_slab_outer);
         else if(q->elem_bytes == 16)
             hipLaunchKernelGGL(probe_tiles<v4f>, dim3(grid), dim3(256), 0, s, static_cast<const v4f*>(q->src),
                                static_cast<v4f*>(q->dst), W, q->in_row, q->out_row, q->tiles_per_slab, q->in_slab,
-                               q->out_slab, (uint32_t)total, q->nontemporal, xcd);
+                               q->out_slab, (uint32_t)total, q->nontemporal, xcd, q->slabs_inner, q->in_slab_outer,
+                               q->out_slab_outer);
         else
             return (int)hipErrorInvalidValue;
         break;

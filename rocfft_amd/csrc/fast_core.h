@@ -529,14 +529,14 @@ FFT_DEV uint32_t fk_w_out(const fftk_params& p, const TileCtx<T>& c, uint32_t w)
 
 // The large twiddles W_L^{j q} of a thread's outputs j = ot + s TPT + k CL of the last pass, in
 // factored form: W^{q ot} . W^{q s TPT} . W^{q (k mod 4) CL} . W^{q 4 (k div 4) CL} (the last two
-// as one factor when the radix is no multiple of 4).  A thread with S x R outputs looks up
-// 1 + (S-1) + 3 + (R/4-1) table values instead of S R of them -- 7 instead of 16 for 64 points
-// in 4 threads, or for one radix-16 butterfly a thread -- and every twiddle is the product of
-// at most four table values, each the product of the two entries of the two-level table.  The
-// lookups depend only on the thread's place in the tile, so a kernel can issue them before it
-// loads its data (fetch) and form the table values while the data is on its way (combine);
-// the dependent round trip to the tables then no longer sits between the last butterfly and
-// the stores.
+// as one factor for radices up to 4).  A thread with S x R outputs looks up
+// 1 + (S-1) + 3 + (ceil(R/4)-1) table values instead of S R of them -- 7 instead of 16 for 64
+// points in 4 threads, or for one radix-16 butterfly a thread; 8 instead of 17 for radix 17 --
+// and every twiddle is the product of at most four table values, each the product of the two
+// entries of the two-level table.  The lookups depend only on the thread's place in the tile,
+// so a kernel can issue them before it loads its data (fetch) and form the table values while
+// the data is on its way (combine); the dependent round trip to the tables then no longer sits
+// between the last butterfly and the stores.
 template <typename T, typename Cfg>
 struct FkStoreTwiddles
 {
@@ -545,9 +545,9 @@ struct FkStoreTwiddles
     static constexpr int              RL     = Cfg::radix(LAST);
     static constexpr int              SL     = Cfg::S(LAST);
     static constexpr int              CL     = Cfg::N / RL;
-    static constexpr bool             SPLITK = RL > 4 && RL % 4 == 0;
+    static constexpr bool             SPLITK = RL > 4;
     static constexpr int              KL     = SPLITK ? 4 : RL;
-    static constexpr int              KH     = SPLITK ? RL / 4 : 1;
+    static constexpr int              KH     = SPLITK ? (RL + 3) / 4 : 1;
     static constexpr int              NL     = 1 + (SL - 1) + (KL - 1) + (KH - 1);
     C                                 f[NL], g[NL];
     FFT_DEV void fetch(const fftk_params& p, uint32_t ot, uint32_t oq)

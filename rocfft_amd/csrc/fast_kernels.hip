@@ -123,13 +123,18 @@ __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
 }
 
 // Which variants request the table values of the large twiddle on the store side before their
-// data: those with registers to spare for them.  Double-precision kernels hold 64 registers of
-// data and 60 of pass twiddles; the 7 table values (28 registers) fit into the first pass of a
-// chirp-z transform up to 512 points, beyond that the kernels spill.
+// data: those with registers to spare for them.  The variant for twiddled passes does so for
+// powers of two (7 table values at most; the other lengths run other kinds of passes on this
+// variant as well, the tile copy of short transforms among them, and the registers the early
+// values hold cost those an occupancy step: 100 points went from 63 to 100 registers, 17 points
+// spilled).  Double-precision kernels hold 64 registers of data and 60 of pass twiddles; the 7
+// table values (28 registers) fit into the first pass of a chirp-z transform up to 512 points,
+// beyond that the kernels spill.
 template <typename T, typename Cfg, int MODE>
 constexpr bool fast_early_twiddles()
 {
-    return MODE == 4 || ((MODE == 7 || MODE == 9) && (sizeof(T) == 4 || (MODE == 7 && Cfg::N <= 512)));
+    constexpr bool pow2 = (Cfg::N & (Cfg::N - 1)) == 0;
+    return (MODE == 4 && pow2) || ((MODE == 7 || MODE == 9) && (sizeof(T) == 4 || (MODE == 7 && Cfg::N <= 512)));
 }
 
 template <typename T, typename Cfg, int MODE>

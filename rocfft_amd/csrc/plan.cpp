@@ -2308,12 +2308,12 @@ static void emit_real_step(Builder& b, PassKind kind, uint64_t half, const std::
 
 // A single-pass dimension d followed by a long strided dimension e = d+1 (a "column"
 // dimension too long for one column tile, e.g. the second dimension of a 4096 x 4096
-// transform).  Power-of-two strides between the rows of such an array alias onto the same
-// HBM channel and bank, so reading stride-n0 rows of the user's array runs at a fraction of
-// the streaming rate.  The pass over d therefore writes its rows into the work buffer in
-// permuted order (row n1*n0 + n0' of dimension e goes to slot n0'*n1 + n1) with a padded
-// row pitch: pass A of the split then reads n1 consecutive rows, and pass B reads rows that
-// are a non-power-of-two stride apart before writing the user's output.
+// transform).  The pass over d writes its rows into the work buffer in permuted order (row
+// n1*n0 + n0' of dimension e goes to slot n0'*n1 + n1): pass A of the split then reads n1
+// consecutive rows where the plain split reads rows n0 apart, and pass B reads the strided rows
+// before writing the user's output.  Measured on MI355X against the plain split of the same
+// lengths: 4096 x 4096 x 8 single precision 1.23 against 1.28 ms, the other shapes tried
+// (2048^2 ... 8192^2, 512 x 16384, both precisions) within 3 % either way.
 static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t batch, size_t d,
                              const View& src, const View& out, int dir, const DimOps& last_ops)
 {
@@ -2361,12 +2361,15 @@ static bool emit_dims_staged(Builder& b, const size_t* len, size_t rank, size_t 
         tstride[i] = run;
         run *= (int64_t)len[i];
     }
-    // Padded pitch between the rows of dimension e: 512 bytes more than a row (measured on the
-    // 4096 x 4096 single-precision transform: no padding, pass B 0.435 ms; 256 bytes, 0.488 ms --
-    // every other row then starts in the middle of a 512-byte block; 512 bytes, 0.408 ms; 1 KB,
-    // 0.416 ms; 4 KB, 0.441 ms).  ROCFFT_AMD_STAGE_PAD sets it in scalars (comparisons).
+    // Pitch between the rows of dimension e: the row itself, no padding.  Sum of pass A and B over
+    // paddings of 0 / 128 / 256 / 512 / 1024 bytes, MI355X: 4096 x 4096 x 8 single 0.803 / 0.821 /
+    // 0.882 / 0.808 / 0.827 ms; 8192 x 8192 single 0.406 / 0.408 / 0.411 / 0.517 / 0.411;
+    // 4096 x 4096 x 4 double 0.846 / 0.831 / 0.824 / 0.970 / 0.840; 8192 x 8192 double 0.807 / 0.806 /
+    // 0.804 / 0.820 / 1.092: every padding tried is the slow one for some shape (rows that come to
+    // lie 2^k + 32 KiB apart), the power-of-two pitch for none of fourteen.
+    // ROCFFT_AMD_STAGE_PAD sets the padding in scalars (comparisons).
     static const char* pad_env = getenv("ROCFFT_AMD_STAGE_PAD");
-    const int64_t      rowS    = run + (pad_env ? atol(pad_env) : (int64_t)(512 / (esize / 2)));
+    const int64_t      rowS    = run + (pad_env ? atol(pad_env) : 0);
     const int64_t      s_n1 = rowS, s_n0 = (int64_t)n1 * rowS;
     run                = (int64_t)n0 * s_n0;
     for(size_t i = e + 1; i < rank; ++i)
