@@ -2958,6 +2958,10 @@ void half_scratch_needs(const ExecPlan& plan, bool fuse_in, bool fuse_out, bool&
 // side starts and ends on a 128-byte line: on tiles that share lines with their neighbours the
 // hint keeps the halves from merging in the cache (512 x 512 x 257 double-precision columns,
 // 257 bins a row: 0.43 -> 0.84 ms), and double-precision passes measured 3-8 % slower with it.
+// And only where every access of a wave covers whole lines: along a transform the lanes of one
+// transform read neighbouring elements, so with fewer than 128 bytes of lanes a transform a line
+// is fetched piecewise by several instructions, and with the hint once for each of them (rows
+// of 32 points, 2 threads a transform, 1 GB: 0.48 -> 2.65 ms).
 static const double NT_MIN_MBYTES = 768.0;
 static bool pass_streams_side(const fftk_params& k, bool in)
 {
@@ -2972,7 +2976,10 @@ static bool pass_streams_side(const fftk_params& k, bool in)
             return false;
     if(fast_tile) // runs of W elements along the tile axis
         return w == 2 && (k.W * 2) % line == 0 && t % line == 0 && k.tile_cnt % k.W == 0;
-    // runs of n elements along the transform
+    // runs of n elements along the transform, T lanes of a transform side by side (or the tile
+    // copied through LDS by consecutive lanes)
+    if(!k.stage_io && ((int64_t)k.T * 2) % line)
+        return false;
     return t == 2 && ((int64_t)k.n * 2) % line == 0 && (k.tile_cnt == 1 || w % line == 0);
 }
 
