@@ -452,6 +452,9 @@ def copy_probes():
         # configuration 2: one workgroup of 1024 threads per row of 256 KiB
         "rows of 32768, 32 loads then 32 stores, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=32, workgroups_per_cu=1),
         "rows of 32768, 8 loads then 8 stores, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=8, workgroups_per_cu=1),
+        "rows of 32768, 4 loads then 4 stores, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=4, workgroups_per_cu=1),
+        "rows of 32768, 2 loads then 2 stores, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=2, workgroups_per_cu=1),
+        "rows of 32768, 1 load then 1 store, 1 workgroup per CU": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32768, group=1, workgroups_per_cu=1),
         "rows of 32768 read, rows 32769 apart written (real forward), 32/32": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32769, group=32, workgroups_per_cu=1),
         "rows 32769 apart read, rows of 32768 written (real inverse), 32/32": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32769, out_row=32768, group=32, workgroups_per_cu=1),
         "rows 32769 apart written, 8/8": dict(shape=B.PROBE_ROWS, rows=rows, in_row=32768, out_row=32769, group=8, workgroups_per_cu=1),

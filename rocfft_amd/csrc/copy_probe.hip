@@ -173,12 +173,21 @@ extern "C" int fftrt_copy_probe(const struct rocfft_amd_probe* q, void* stream)
         if(!q->src || q->rows == 0 || q->in_row < 32768 || q->out_row < 32768)
             return (int)hipErrorInvalidValue;
         const uint32_t grid = std::min<uint32_t>(q->rows, per_cu * (uint32_t)cus);
-        if(q->group == 8)
-            hipLaunchKernelGGL(probe_rows<8>, dim3(grid), dim3(1024), 0, s, static_cast<const v2f*>(q->src),
-                               static_cast<v2f*>(q->dst), q->in_row, q->out_row, q->rows, q->nontemporal);
-        else
-            hipLaunchKernelGGL(probe_rows<32>, dim3(grid), dim3(1024), 0, s, static_cast<const v2f*>(q->src),
-                               static_cast<v2f*>(q->dst), q->in_row, q->out_row, q->rows, q->nontemporal);
+        const v2f* src = static_cast<const v2f*>(q->src);
+        v2f*       dst = static_cast<v2f*>(q->dst);
+#define PROBE_ROWS_GROUP(G)                                                                                      \
+    hipLaunchKernelGGL(probe_rows<G>, dim3(grid), dim3(1024), 0, s, src, dst, q->in_row, q->out_row, q->rows, \
+                       q->nontemporal)
+        switch(q->group)
+        {
+        case 1: PROBE_ROWS_GROUP(1); break;
+        case 2: PROBE_ROWS_GROUP(2); break;
+        case 4: PROBE_ROWS_GROUP(4); break;
+        case 8: PROBE_ROWS_GROUP(8); break;
+        case 16: PROBE_ROWS_GROUP(16); break;
+        default: PROBE_ROWS_GROUP(32); break;
+        }
+#undef PROBE_ROWS_GROUP
         break;
     }
     case ROCFFT_AMD_PROBE_TILES:
