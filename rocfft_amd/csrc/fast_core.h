@@ -702,7 +702,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
             // (entries beyond the tile read the table at index 0)
             const bool     in_tile = active && (c.tile0 + ow0 < p.tile_cnt);
             const uint32_t oq0     = p.aux_dim == 1 ? (c.tile0 + ow0) >> p.aux_shift : c.q_block;
-            stw.fetch(p, in_tile ? ot0 : 0u, in_tile ? oq0 : 0u);
+            stw.fetch(p, in_tile ? ot0 : 0u, in_tile ? oq0 * p.ltw_qmul + p.ltw_qadd : 0u);
         }
     }
     // ---------------------------------------------------------------- load
@@ -1331,7 +1331,7 @@ __device__ __forceinline__ void fast_tile_lean(const fftk_params& p, typename cp
         {
             if constexpr(!EARLY_TW)
             {
-                stw.fetch(p, ot, oq);
+                stw.fetch(p, ot, oq * p.ltw_qmul + p.ltw_qadd);
                 stw.combine();
             }
 #pragma unroll

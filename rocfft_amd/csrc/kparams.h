@@ -119,6 +119,7 @@ struct fftk_params
     const void* convb;     // spectrum the tile is multiplied with in CONV mode
     const void* tw2;       // fused 2D kernel: stacked twiddles of the second dimension
     uint32_t    ltw_shift; //
+    uint32_t    ltw_qmul, ltw_qadd; // the large twiddle of output j is W_L^{j (q ltw_qmul + ltw_qadd)}
     uint32_t    blu_n;
     uint32_t    chirp_js, chirp_qs; // logical sample index = j*chirp_js + q*chirp_qs
     uint32_t    convb_qs;           // convb index = j + q*convb_qs

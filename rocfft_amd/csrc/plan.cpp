@@ -605,7 +605,9 @@ struct TileSpec
     uint32_t          n_in = 0, n_out = 0; // 0 = n
     TablePtr          ltw, half_tw, chirp, convb;
     uint32_t          ltw_shift = 0;
+    uint32_t          ltw_qmul = 1, ltw_qadd = 0; // twiddle of output j: W^{j (q ltw_qmul + ltw_qadd)}
     uint32_t          blu_n = 0, chirp_js = 0, chirp_qs = 0, convb_qs = 0;
+    uint64_t          convb_off = 0; // first element of the chirp spectrum this pass reads
     double            scale = 1.0;
     std::string       note;
     bool              src_real_scalar = false, dst_real_scalar = false;
@@ -882,6 +884,8 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     {
         k.ltw       = s.ltw->dptr;
         k.ltw_shift = s.ltw_shift;
+        k.ltw_qmul  = s.ltw_qmul;
+        k.ltw_qadd  = s.ltw_qadd;
         rec.tables.push_back(s.ltw);
     }
     if(s.half_tw)
@@ -899,7 +903,7 @@ static PassRec make_tile_pass(const TileSpec& s, int precision, bool dry)
     }
     if(s.convb)
     {
-        k.convb    = s.convb->dptr;
+        k.convb    = s.convb->dptr ? static_cast<const char*>(s.convb->dptr) + s.convb_off * esize : nullptr;
         k.convb_qs = s.convb_qs;
         rec.tables.push_back(s.convb);
     }
@@ -1296,7 +1300,7 @@ static bool smooth(uint64_t n)
 }
 
 static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t M1, uint64_t M0,
-                                   bool conj_chirp);
+                                   bool conj_chirp, uint64_t M2 = 1);
 static bool     big_eligible(const Builder& b, uint64_t n, int64_t t_is, int64_t t_os,
                              const std::vector<Other>& others, const IoRef& src, const IoRef& dst);
 static void     emit_big(Builder& b, uint32_t mode, const std::vector<Other>& others, const IoRef& src,
@@ -1633,7 +1637,7 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     }
     bool one = sM1 == 0 && one_kernel(M);
     // single precision: the wide compiled kernels (up to M = 16384) still fit one workgroup
-    const bool wide_one = sM1 == 0 && !one && !column && wide_kernel_length(M, esize);
+    bool wide_one = sM1 == 0 && !one && !column && wide_kernel_length(M, esize);
     // (checked before any table is computed: a chirp of 10^8 entries takes a minute)
     if(!one && !wide_one && (ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out))
         fail("odd-length real transforms of this size are not implemented");
@@ -1642,7 +1646,38 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     uint64_t row_len = 4096;
     if(!one && sM1 == 0 && !single_kernel_length(M / row_len, esize) && single_kernel_length(8192, esize))
         row_len = 8192;
-    if(!one && sM1 == 0 && !single_kernel_length(M / row_len, esize))
+    // Beyond row_len^2 points (2^26) the strided factor no longer fits one kernel either: three
+    // levels, M = M2 * M1 * M0 (below).  ROCFFT_AMD_BLU3=<m1>,<m0> forces that form with these two
+    // factors at any length they divide (tests, comparisons).
+    uint64_t M2 = 0, f1 = 0, f0 = 0;
+    {
+        const char*        env = getenv("ROCFFT_AMD_BLU3");
+        unsigned long long a = 0, c = 0;
+        if(env && sscanf(env, "%llu,%llu", &a, &c) == 2 && a > 1 && c > 1 && Mpow2 % (a * c) == 0 && Mpow2 / (a * c) > 1)
+        {
+            M   = Mpow2;
+            sM1 = sM0 = 0;
+            one       = false;
+            f1        = a;
+            f0        = c;
+            M2        = M / (a * c);
+            wide_one  = false;
+        }
+    }
+    if(M2 == 0 && !one && sM1 == 0 && !single_kernel_length(M / row_len, esize))
+    {
+        // rows of 4096 points; the middle factor as long as a strided pass with full tile rows
+        // takes (fewer launches of the row kernel), the rest to the outer factor
+        f0 = 4096;
+        for(f1 = 4096; f1 >= 64; f1 /= 2)
+            if(column_kernel_length(f1, esize) && M / (f1 * f0) >= 2 && column_kernel_length(M / (f1 * f0), esize))
+                break;
+        if(f1 < 64)
+            fail("Bluestein length too large");
+        M2 = M / (f1 * f0);
+    }
+    if(M2 != 0
+       && !(M2 >= 2 && column_kernel_length(M2, esize) && column_kernel_length(f1, esize) && single_kernel_length(f0, esize)))
         fail("Bluestein length too large");
     TablePtr chirp      = chirp_table(N, b.precision, b.dry);
     double   scale      = (1.0 / (double)M) * (ops.has_scale ? ops.scale : 1.0);
@@ -1706,6 +1741,140 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
     }
     if(ops.load_op == FFTK_LOAD_HERM_EXPAND || ops.n_out)
         fail("odd-length real transforms of this size are not implemented");
+    if(M2 != 0)
+    {
+        // Three levels, M = M2 * M1 * M0, sample n = (n2 M1 + n1) M0 + n0, bin k = k2 + M2 (k1 + M1 k0):
+        //   P1  chirp, pad, FFT over n2 (stride M1 M0), times W_M^{k2 (n1 M0 + n0)}            [like Z1]
+        //   P2  in every block k2: FFT over n1 (stride M0), times W_{M1 M0}^{k1 n0}
+        //   P3  one launch per block k2: every row (k2, k1) is transformed over n0, multiplied by
+        //       its row of the chirp spectrum (kept in this order), transformed back and multiplied
+        //       by conj W_M^{n0 (M2 k1 + k2)} -- the twiddle of the inverse over k1 and the part
+        //       W_M^{k2 n0} of the twiddle of the inverse over k2, which does not depend on n1  [like Z2]
+        //   P4  in every block k2: inverse FFT over k1, times conj W_{M2 M1}^{k2 n1} (the rest of it)
+        //   P5  inverse FFT over k2, chirp, scale, first n outputs                              [like Z3]
+        // The padded signals are M contiguous elements each (no row padding: the tile axis of P1 and
+        // P5 runs over n1 and n0 together).
+        const uint64_t M1 = f1, M0 = f0, R = M1 * M0;
+        TablePtr bs = bluestein_spectrum(b, N, M, M1, M0, conj_chirp, M2);
+        std::vector<int64_t> pk(others.size(), 0);
+        int64_t              inner = 1;
+        {
+            std::vector<size_t> order(others.size());
+            for(size_t i = 0; i < others.size(); ++i)
+                order[i] = i;
+            std::sort(order.begin(), order.end(), [&](size_t x, size_t y) { return others[x].is < others[y].is; });
+            for(size_t i : order)
+                if(column && others[i].cnt > 1 && others[i].is < t_is)
+                {
+                    pk[i] = 2 * inner;
+                    inner *= others[i].cnt;
+                }
+            int64_t outer = (int64_t)M * 2 * inner;
+            for(size_t i : order)
+                if(pk[i] == 0)
+                {
+                    pk[i] = outer;
+                    outer *= others[i].cnt;
+                }
+            b.need_blu((size_t)(outer / 2));
+        }
+        const int64_t qS = 2 * inner;
+        {
+            TileSpec s = base_spec();
+            s.dir      = -1;
+            s.n        = (uint32_t)M2;
+            s.t_is     = (int64_t)R * t_is;
+            s.t_os     = (int64_t)R * qS;
+            s.src      = src;
+            s.dst      = blu;
+            s.others.push_back({(uint32_t)R, t_is, qS, true});
+            add_others(s, true, false, pk);
+            s.load_op         = ops.load_op;
+            s.src_real_scalar = ops.src_real_scalar;
+            s.flags |= FFTK_F_CHIRP_LOAD | FFTK_F_TWIDDLE_STORE | cflag;
+            s.chirp     = chirp;
+            s.blu_n     = (uint32_t)N;
+            s.chirp_js  = (uint32_t)R;
+            s.chirp_qs  = 1;
+            s.ltw       = large_twiddles(M, b.precision, b.dry);
+            s.ltw_shift = large_twiddle_shift(M);
+            s.note      = dims_note("bluestein P1 (chirp, pad, column fft over the outer factor, twiddle)", M2);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        {
+            TileSpec s = base_spec();
+            s.dir      = -1;
+            s.n        = (uint32_t)M1;
+            s.t_is = s.t_os = (int64_t)M0 * qS;
+            s.src = s.dst = blu;
+            s.others.push_back({(uint32_t)M0, qS, qS, true});
+            s.others.push_back({(uint32_t)M2, (int64_t)R * qS, (int64_t)R * qS, false});
+            add_others(s, false, false, pk);
+            s.flags |= FFTK_F_TWIDDLE_STORE;
+            s.ltw       = large_twiddles(R, b.precision, b.dry);
+            s.ltw_shift = large_twiddle_shift(R);
+            s.note      = dims_note("bluestein P2 (column fft over the middle factor, twiddle)", M1);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        for(uint64_t k2 = 0; k2 < M2; ++k2)
+        {
+            TileSpec s = base_spec();
+            s.dir      = -1;
+            s.n        = (uint32_t)M0;
+            s.t_is = s.t_os = qS;
+            s.src = s.dst = blu;
+            s.src_extra = s.dst_extra = (int64_t)(k2 * R) * qS;
+            s.others.push_back({(uint32_t)M1, (int64_t)M0 * qS, (int64_t)M0 * qS, true});
+            add_others(s, false, false, pk);
+            s.flags |= FFTK_F_CONV | FFTK_F_TWIDDLE_STORE;
+            s.convb     = bs;
+            s.convb_qs  = (uint32_t)M0;
+            s.convb_off = k2 * R;
+            s.ltw       = large_twiddles(M, b.precision, b.dry);
+            s.ltw_shift = large_twiddle_shift(M);
+            s.ltw_qmul  = (uint32_t)M2;
+            s.ltw_qadd  = (uint32_t)k2;
+            s.note      = dims_note("bluestein P3 (rows of one block: fft, multiply, inverse fft, twiddle)", M0);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        {
+            TileSpec s = base_spec();
+            s.dir      = +1;
+            s.n        = (uint32_t)M1;
+            s.t_is = s.t_os = (int64_t)M0 * qS;
+            s.src = s.dst = blu;
+            s.others.push_back({(uint32_t)M0, qS, qS, false});
+            s.others.push_back({(uint32_t)M2, (int64_t)R * qS, (int64_t)R * qS, true});
+            add_others(s, false, false, pk);
+            s.flags |= FFTK_F_TWIDDLE_STORE;
+            s.ltw       = large_twiddles(M2 * M1, b.precision, b.dry);
+            s.ltw_shift = large_twiddle_shift(M2 * M1);
+            s.note      = dims_note("bluestein P4 (inverse column fft over the middle factor, twiddle)", M1);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        {
+            TileSpec s = base_spec();
+            s.dir      = +1;
+            s.n        = (uint32_t)M2;
+            s.t_is     = (int64_t)R * qS;
+            s.t_os     = (int64_t)R * t_os;
+            s.src      = blu;
+            s.dst      = dst;
+            s.others.push_back({(uint32_t)R, qS, t_os, true});
+            add_others(s, false, true, pk);
+            s.store_op        = ops.store_op;
+            s.dst_real_scalar = ops.dst_real_scalar;
+            s.flags |= FFTK_F_CHIRP_STORE | FFTK_F_SCALE | cflag;
+            s.chirp    = chirp;
+            s.blu_n    = (uint32_t)N;
+            s.chirp_js = (uint32_t)R;
+            s.chirp_qs = 1;
+            s.scale    = scale;
+            s.note     = dims_note("bluestein P5 (inverse column fft over the outer factor, chirp, scale)", M2);
+            b.plan->passes.push_back(make_tile_pass(s, b.precision, b.dry));
+        }
+        return;
+    }
     // M = M1*M0: rows of length M0 are transformed, multiplied and transformed back by
     // one kernel, so that kernel gets the long factor; the strided passes get M1
     uint64_t M0 = row_len, M1 = M / M0;
@@ -1830,10 +1999,10 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
 // library's own passes and narrowed to the plan precision.  For a split M the
 // result is kept in the order the convolution kernel meets it: [k1*M0 + k0].
 static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t M1, uint64_t M0,
-                                   bool conj_chirp)
+                                   bool conj_chirp, uint64_t M2)
 {
     std::ostringstream key;
-    key << "bspec_" << N << "_" << M << "_" << M1 << "_" << M0 << (conj_chirp ? "c" : "f");
+    key << "bspec_" << N << "_" << M << "_" << M2 << "_" << M1 << "_" << M0 << (conj_chirp ? "c" : "f");
     int dev = 0;
     if(!b.dry)
         fftrt_device_info(&dev, nullptr, nullptr, nullptr, 0);
@@ -1881,6 +2050,39 @@ static TablePtr bluestein_spectrum(Builder& b, uint64_t N, uint64_t M, uint64_t 
         DimOps none;
         if(M1 == 0)
             emit_dim(sb, M, 2, 2, {}, io, io, -1, none);
+        else if(M2 > 1)
+        {
+            // three levels: the forward passes of the convolution itself, order [k2][k1][k0]
+            const uint64_t R = M1 * M0;
+            TileSpec       a;
+            a.dir  = -1;
+            a.n    = (uint32_t)M2;
+            a.t_is = a.t_os = (int64_t)R * 2;
+            a.src = a.dst = io;
+            a.others.push_back({(uint32_t)R, 2, 2, true});
+            a.flags |= FFTK_F_TWIDDLE_STORE;
+            a.ltw       = large_twiddles(M, 1, false);
+            a.ltw_shift = large_twiddle_shift(M);
+            sub.passes.push_back(make_tile_pass(a, 1, false));
+            TileSpec c;
+            c.dir  = -1;
+            c.n    = (uint32_t)M1;
+            c.t_is = c.t_os = (int64_t)M0 * 2;
+            c.src = c.dst = io;
+            c.others.push_back({(uint32_t)M0, 2, 2, true});
+            c.others.push_back({(uint32_t)M2, (int64_t)R * 2, (int64_t)R * 2, false});
+            c.flags |= FFTK_F_TWIDDLE_STORE;
+            c.ltw       = large_twiddles(R, 1, false);
+            c.ltw_shift = large_twiddle_shift(R);
+            sub.passes.push_back(make_tile_pass(c, 1, false));
+            TileSpec r;
+            r.dir  = -1;
+            r.n    = (uint32_t)M0;
+            r.t_is = r.t_os = 2;
+            r.src = r.dst = io;
+            r.others.push_back({(uint32_t)(M2 * M1), (int64_t)M0 * 2, (int64_t)M0 * 2, false});
+            sub.passes.push_back(make_tile_pass(r, 1, false));
+        }
         else
         {
             TablePtr ltw = large_twiddles(M, 1, false);

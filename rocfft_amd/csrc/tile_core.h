@@ -465,7 +465,7 @@ FFT_DEV void emit_elem(const fftk_params& p, const TileCtx<T>& c, uint32_t w, ui
     uint32_t q = p.aux_dim == 1 ? (c.tile0 + w) >> p.aux_shift : c.q_block;
     if(p.flags & FFTK_F_TWIDDLE_STORE)
     {
-        C t = large_twiddle<T>(p, j * q);
+        C t = large_twiddle<T>(p, j * (q * p.ltw_qmul + p.ltw_qadd));
         v   = inv ? c_mulc(v, t) : c_mul(v, t);
     }
     if(p.flags & FFTK_F_CHIRP_STORE)

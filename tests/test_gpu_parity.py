@@ -284,6 +284,20 @@ def test_four_pass_split(gpu, monkeypatch):
     H.check(lib, be, B.COMPLEX_FORWARD, [2 ** 17], 2, B.DOUBLE)
 
 
+def test_three_level_chirp_z(gpu, monkeypatch):
+    """the chirp-z form for convolution lengths beyond 2^26, asked for at lengths the checker
+    finishes (tests/test_reference_matrix.py runs a prime that needs it)"""
+    lib, be = gpu
+    monkeypatch.setenv("ROCFFT_AMD_BLU3", "64,128")
+    for n in (100003, 1000003):  # 2^18 = 32 x 64 x 128, 2^21 = 256 x 64 x 128
+        H.check(lib, be, B.COMPLEX_FORWARD, [n], 2, B.SINGLE)
+        H.check(lib, be, B.COMPLEX_INVERSE, [n], 1, B.DOUBLE, inplace=True, scale=0.5)
+    monkeypatch.setenv("ROCFFT_AMD_BLU3", "16,4096")
+    H.check(lib, be, B.COMPLEX_FORWARD, [1000003], 3, B.DOUBLE)
+    H.check(lib, be, B.COMPLEX_FORWARD, [7, 100003], 1, B.SINGLE)
+    H.check(lib, be, B.COMPLEX_FORWARD, [100003, 3], 1, B.SINGLE)
+
+
 @pytest.mark.parametrize("lengths", [[8193], [10007], [19683], [15625], [100003], [9999, 3], [3, 9999]])
 def test_long_odd_real(gpu, lengths):
     lib, be = gpu

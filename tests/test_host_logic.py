@@ -308,6 +308,32 @@ def test_four_pass_split(emu, monkeypatch):
     H.check(emu, HOST, B.COMPLEX_FORWARD, [32768], 2, B.SINGLE)
 
 
+def test_three_level_chirp_z(emu, monkeypatch):
+    """A convolution length beyond 2^26 (a prime above 2^25) splits into three factors: two strided
+    passes each way and one launch of the row kernel per block of rows.  ROCFFT_AMD_BLU3=<m1>,<m0>
+    asks for that form at lengths the checker finishes."""
+    st, text, work = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [33554467], 1)
+    assert st == 0, text
+    names = [l for l in passes(text)]
+    assert len(names) == 4 + 64 and sum("bluestein P3" in l for l in names) == 64, text  # 2^27 = 64 x 512 x 4096
+    assert work == 2 ** 27 * 8
+    # the largest convolution length, 2^30
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [400000009], 1)
+    assert st == 0 and text.startswith("plan: 516 passes"), text[:300]  # 2^30 = 512 x 512 x 4096
+    # 2^31 is beyond the 32-bit sample index of the tables
+    st, text, _ = emu.describe(B.NOTINPLACE, B.COMPLEX_FORWARD, B.SINGLE, [536870923], 1)
+    assert st != 0
+    monkeypatch.setenv("ROCFFT_AMD_BLU3", "8,16")
+    for kind, lengths, batch, prec in ((B.COMPLEX_FORWARD, [1009], 3, B.DOUBLE), (B.COMPLEX_INVERSE, [1009], 2, B.SINGLE),
+                                       (B.COMPLEX_FORWARD, [521], 4, B.SINGLE), (B.COMPLEX_FORWARD, [1031], 1, B.DOUBLE),
+                                       (B.COMPLEX_FORWARD, [5, 1009], 2, B.DOUBLE), (B.COMPLEX_FORWARD, [1009, 3], 2, B.SINGLE),
+                                       (B.REAL_FORWARD, [6, 1009], 1, B.DOUBLE)):
+        st, text, _ = emu.describe(B.NOTINPLACE, kind, prec, lengths, batch)
+        assert st == 0 and "bluestein P3" in text and "bluestein P5" in text, text
+        H.check(emu, HOST, kind, lengths, batch, prec)
+        H.check(emu, HOST, kind, lengths, batch, prec, inplace=True, scale=0.5)
+
+
 def test_one_transform_ignores_the_distances(emu):
     """in place, one transform, different input and output distances (the reference's tests do
     this: clients/tests/accuracy_test_adhoc.cpp:84-157)"""

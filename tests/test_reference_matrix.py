@@ -304,6 +304,19 @@ def test_long_lengths_of_the_1d_lists(gpu, n):
     be.torch.cuda.empty_cache()
 
 
+def test_prime_above_2_to_the_25(gpu):
+    """33554467, the first prime above 2^25: its convolution length, 2^27, is beyond two levels of
+    kernels (the reference takes any prime that fits memory, library/src/tree_node_bluestein.cpp:27-285);
+    planned as 64 x 512 x 4096 with one launch of the row kernel per block of 512 rows"""
+    lib, be = gpu
+    n = 33554467
+    print("prime", n, flush=True)
+    _spot_check_1d(lib, be, n, B.SINGLE)
+    be.torch.cuda.empty_cache()
+    _closed_forms_1d(lib, be, n, B.SINGLE)
+    be.torch.cuda.empty_cache()
+
+
 # clients/tests/accuracy_test_adhoc.cpp:25-60 (slowest dimension first)
 ADHOC_SIZES = [[1, 220], [1, 330], [81, 220, 36], [4, 4, 8192], [192, 192, 192], [192, 84, 84], [680, 128, 128],
                [196597], [25165813], [19, 2053], [98, 98, 98], [336, 336, 56]]
