@@ -27,8 +27,10 @@ namespace
 // scale factor); 4: interleaved arrays, a scale factor, the large twiddle on the store side, the
 // fused real pre/post-processing, the tile copy of short transforms, and (single precision)
 // arrays of IEEE half pairs on the load or the store side: the first and last pass of a
-// half-precision plan, which computes in single precision; 7, 9 and 8: the first, middle and last
-// pass of a chirp-z transform in three kernels (powers of two only).  The variants 3, 4, 7, 8, 9 are
+// half-precision plan, which computes in single precision; 5 (odd lengths): real samples on one
+// side and the half spectrum on the other, nothing else fused but a scale factor; 7, 9 and 8: the
+// first, middle and last pass of a chirp-z transform in three kernels (powers of two only).  The
+// variants 3, 4, 5, 7, 8, 9 are
 // the lean kernel compiled under assumptions on its arguments (fast_assume_plain): the compiler
 // drops every other path, which leaves a fifth to a third of the code and 10-50 registers fewer.
 // Workgroups have up to 512 threads (row passes use up to 256, strided passes more to keep
@@ -52,6 +54,21 @@ __device__ __forceinline__ void fast_assume_plain(const fftk_params& p)
         __builtin_assume(p.in_planar == 0);
         __builtin_assume(p.out_planar == 0);
         __builtin_assume(p.w_inner == 0);
+    }
+    else if constexpr(MODE == 5)
+    {
+        // odd-length real transforms: real samples -> half spectrum, or half spectrum -> real samples
+        __builtin_assume(p.load_op == FFTK_LOAD_REAL || p.load_op == FFTK_LOAD_HERM_EXPAND);
+        __builtin_assume(p.store_op == FFTK_STORE_COMPLEX || p.store_op == FFTK_STORE_REAL);
+        __builtin_assume((p.flags & ~(uint32_t)FFTK_F_SCALE) == 0);
+        __builtin_assume(p.in_planar == 0);
+        __builtin_assume(p.out_planar == 0);
+        __builtin_assume(p.stage_io == 0);
+        __builtin_assume(p.w_inner == 0);
+        __builtin_assume(p.aux_dim == 0);
+        __builtin_assume(p.oc0_first == 0);
+        __builtin_assume(p.in_nt == 0);
+        __builtin_assume(p.out_nt == 0);
     }
     else if constexpr(MODE == 7)
     {
@@ -166,7 +183,7 @@ __global__ __launch_bounds__(fast_block_limit<Cfg>(), WAVES) void fast_tile_kern
 template <typename T, typename Cfg, int MODE>
 constexpr int fast_waves()
 {
-    return (sizeof(T) == 4 && (MODE == 3 || MODE == 4) && Cfg::TPT <= 512) ? 4 : 0;
+    return (sizeof(T) == 4 && (MODE == 3 || MODE == 4 || MODE == 5) && Cfg::TPT <= 512) ? 4 : 0;
 }
 
 template <typename T, typename Cfg, int MODE>
@@ -217,12 +234,13 @@ constexpr FastEntry fast_entry()
                          fast_variant<T, Cfg, 0, ALL_MODES != 0>(),
                          &launch_fast<T, Cfg, 3>,
                          fast_variant<T, Cfg, 4, more>(),
+                         fast_variant<T, Cfg, 5, Cfg::N % 2 == 1 && (Cfg::N > 1)>(),
                          fast_variant<T, Cfg, 7, ALL_MODES != 0>(),
                          fast_variant<T, Cfg, 8, ALL_MODES != 0>(),
                          fast_variant<T, Cfg, 9, ALL_MODES != 0>()};
     }
     else
-        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+        return FastEntry{-1, 0, {1, 1, 1, 1}, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 }
 
 #define FAST_SCHED(SLICE, FULL, N, A, B, C, D, TTF, TTD, DBL)                  \
@@ -367,6 +385,10 @@ extern "C" int fftrt_launch_fast_tile(const struct fftk_params* p, int precision
                 && (p->load_op == FFTK_LOAD_COMPLEX || p->load_op == FFTK_LOAD_C2R_PRE)
                 && (p->store_op == FFTK_STORE_COMPLEX || p->store_op == FFTK_STORE_R2C_POST))
             fn = e->more;
+        else if(e->odd_real && only_scale && !p->stage_io
+                && ((p->load_op == FFTK_LOAD_REAL && p->store_op == FFTK_STORE_COMPLEX)
+                    || (p->load_op == FFTK_LOAD_HERM_EXPAND && p->store_op == FFTK_STORE_REAL)))
+            fn = e->odd_real;
     }
     // the first and last pass of a chirp-z transform in three kernels (kernels of their own, so
     // that a profile tells them apart)

@@ -23,6 +23,9 @@ struct FastEntry
     // arrays without a chirp (twiddle on the store side, real pre/post-processing, tile copies,
     // half-precision arrays on the user's side)
     fast_launch_fn plain, more;
+    // the lean kernel compiled for odd-length real transforms (real samples on one side, the half
+    // spectrum on the other; odd lengths only)
+    fast_launch_fn odd_real;
     // the lean kernel compiled for the first (chirp and padding on the load side, large twiddle on
     // the store side), the last (chirp and scale on the store side) and the middle pass (forward
     // transform, spectrum product, inverse transform, large twiddle) of a chirp-z transform in
