@@ -127,10 +127,17 @@ class Step:
         return rows
 
 
-def time_steps(torch, step, warmup, steps):
+def time_steps(torch, step, warmup, steps, settle_ms=0.0):
+    """`warmup` untimed steps (and, where asked for, as many more as it takes to fill settle_ms of
+    wall time: the short configurations do not reach settled clocks in 30 steps), then `steps` timed"""
+    t_begin = time.perf_counter()
     for _ in range(warmup):
         step.run()
     torch.cuda.synchronize()
+    while (time.perf_counter() - t_begin) * 1e3 < settle_ms:
+        for _ in range(10):
+            step.run()
+        torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -350,7 +357,7 @@ def reference_child(path, warmup, steps):
     for cid in sorted(wls):
         try:
             step = Step(cid, wls[cid], torch, stream_ptr, lib=lib)
-            ms, _ = time_steps(torch, step, warmup, steps)
+            ms, _ = time_steps(torch, step, warmup, steps, EXTRA_SETTLE_MS)
             out["ms"][wls[cid]["name"]] = ms
             del step
             torch.cuda.empty_cache()
@@ -531,13 +538,14 @@ SHAPE_OF_CONFIG = {
 }
 
 
-# warm-up and timed steps of the other configurations and of the reference library
-EXTRA_WARMUP, EXTRA_STEPS = 30, 20
+# warm-up and timed steps of the other configurations and of the reference library; their warm-up
+# lasts 30 ms at least (30 steps of configuration 1 are 0.5 ms)
+EXTRA_WARMUP, EXTRA_STEPS, EXTRA_SETTLE_MS = 30, 20, 30.0
 
 
-def measure_config(torch, cfg_id, wl, stream_ptr, warmup, steps, prof_reps):
+def measure_config(torch, cfg_id, wl, stream_ptr, warmup, steps, prof_reps, settle_ms=0.0):
     step = Step(cfg_id, wl, torch, stream_ptr)
-    ms, dev_ms = time_steps(torch, step, warmup, steps)
+    ms, dev_ms = time_steps(torch, step, warmup, steps, settle_ms)
     prof = kernel_profile(step, prof_reps)
     return step, ms, dev_ms, prof
 
@@ -663,7 +671,7 @@ def main():
             else:
                 del step
                 torch.cuda.empty_cache()
-                s2, m2, _, p2 = measure_config(torch, cid, wls[cid], stream_ptr, EXTRA_WARMUP, EXTRA_STEPS, 2)
+                s2, m2, _, p2 = measure_config(torch, cid, wls[cid], stream_ptr, EXTRA_WARMUP, EXTRA_STEPS, 2, EXTRA_SETTLE_MS)
                 t2 = torch_fft_ms(torch, cid, s2)
                 step = s2
             w2 = wls[cid]
