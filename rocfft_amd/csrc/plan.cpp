@@ -1664,7 +1664,14 @@ static void emit_dim(Builder& b, uint64_t n, int64_t t_is, int64_t t_os, const s
             wide_one  = false;
         }
     }
-    if(M2 == 0 && !one && sM1 == 0 && !single_kernel_length(M / row_len, esize))
+    // ... and well before that the strided passes of the two-level form, whose tiles hold whole
+    // columns of M / 4096 points, are down to rows of 8 or 16 bytes.  Measured on MI355X, two
+    // levels against three (single precision, one transform): M = 2^24 0.79 against 0.40 ms,
+    // 2^25 2.10 against 0.83 ms, 2^26 2.85 against 1.62 ms (double precision 0.94 / 0.72, 2.46 / 1.38,
+    // 4.35 / 2.61 ms); with two transforms M = 2^24 is a tie (0.76 ms both, double precision 1.16
+    // against 1.31 ms) and below that two levels win (2^23 x 4: 0.62 against 0.73 ms).
+    const bool long_columns = M / 4096 >= 8192 || (M / 4096 >= 4096 && lines == 1);
+    if(M2 == 0 && !one && !wide_one && sM1 == 0 && (long_columns || !single_kernel_length(M / row_len, esize)))
     {
         // rows of 4096 points; the middle factor as long as a strided pass with full tile rows
         // takes (fewer launches of the row kernel), the rest to the outer factor
